@@ -56,8 +56,11 @@ def get_architecture(name: str) -> Architecture:
 
 def architecture_of(config_dict: dict) -> Architecture:
     archs = config_dict.get("architectures")
+    if archs is None and isinstance(config_dict.get("architecture"), str):
+        return get_architecture(config_dict["architecture"])      # some designs name themselves in one string
     if not isinstance(archs, list) or not archs or not isinstance(archs[0], str):
-        raise ConfigError("config.json must name the model in 'architectures' (a non-empty list of strings)")
+        raise ConfigError("config.json must name the model in 'architectures' (a non-empty list of strings) "
+                          "or in 'architecture' (a string)")
     return get_architecture(archs[0])
 
 

@@ -33,6 +33,8 @@ SOURCES = {
     "gemm": "gemm.hip",
     "gemm_mid": "gemm_mid.hip",
     "gemm_wide": "gemm_wide.hip",
+    "latent": "latent.hip",
+    "grouped": "grouped.hip",
     "sampling": "sampling.hip",
     "ceilings": "ceilings.hip",
     "host": "host/api.cpp",

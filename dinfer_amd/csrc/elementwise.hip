@@ -105,6 +105,39 @@ inline unsigned blocks_for(int64_t n, int per_block, unsigned cap) {
   return (unsigned)(b > cap ? cap : b);
 }
 
+// out[t] = table[id] * scale with types of their own: a bf16 table may feed a float residual stream.
+template <class S, class O>
+__global__ void __launch_bounds__(256) embedding_to_kernel(const int32_t* __restrict__ ids, const S* __restrict__ table,
+                                                           O* __restrict__ out, int64_t vocab, int64_t width, float scale,
+                                                           const int32_t* __restrict__ from,
+                                                           const int32_t* __restrict__ last) {
+  const int64_t t = blockIdx.x;
+  int64_t id = ids[t];
+  if (from) {
+    const int32_t at = from[t];
+    if (at >= 0) id = last[at];
+  }
+  if (id < 0 || id >= vocab) id = 0;
+  const S* src = table + id * width;
+  O* dst = out + t * width;
+  for (int64_t i = threadIdx.x; i < width; i += blockDim.x) dst[i] = from_f32<O>(to_f32(src[i]) * scale);
+}
+
+// Activations of one argument: 0 silu, 1 the square of relu, 2 gelu in its tanh form.
+__device__ __forceinline__ float act1(float z, int act) {
+  if (act == 0) return z / (1.f + expf(-z));
+  if (act == 1) { const float r = fmaxf(z, 0.f); return r * r; }
+  return 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+}
+
+template <class S>
+__global__ void __launch_bounds__(256) act_kernel(const S* __restrict__ in, int64_t ld_in, S* __restrict__ out,
+                                                  int64_t ld_out, int64_t n, int act) {
+  const int64_t t = blockIdx.y;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
+    out[t * ld_out + i] = from_f32<S>(act1(to_f32(in[t * ld_in + i]), act));
+}
+
 }  // namespace
 
 // src, last (both or neither): where src[t] >= 0, token t's id is last[src[t]] instead of ids[t].
@@ -178,5 +211,38 @@ extern "C" int dinfer_widen(int dtype, const void* src, float* dst, int64_t n, h
 extern "C" int dinfer_fill_u32(void* dst, uint32_t value, int64_t n_words, hipStream_t stream) {
   if (n_words <= 0) return OK;
   fill_u32_kernel<<<blocks_for(n_words, 256, 4096), 256, 0, stream>>>((uint32_t*)dst, value, n_words);
+  return launch_status();
+}
+
+extern "C" int dinfer_embedding_to(int table_dtype, int out_dtype, const int32_t* ids, const void* table, void* out,
+                                   int64_t tokens, int64_t vocab, int64_t width, float scale, const int32_t* src,
+                                   const int32_t* last, hipStream_t stream) {
+  if (tokens <= 0) return OK;
+  if (vocab <= 0 || width <= 0 || tokens > 0x7fffffff || (!src != !last)) return ERR_BAD_SHAPE;
+  const unsigned g = (unsigned)tokens;
+  if (table_dtype == DT_BF16 && out_dtype == DT_F32)
+    embedding_to_kernel<bf16, float><<<g, 256, 0, stream>>>(ids, (const bf16*)table, (float*)out, vocab, width, scale, src, last);
+  else if (table_dtype == DT_BF16 && out_dtype == DT_BF16)
+    embedding_to_kernel<bf16, bf16><<<g, 256, 0, stream>>>(ids, (const bf16*)table, (bf16*)out, vocab, width, scale, src, last);
+  else if (table_dtype == DT_F32 && out_dtype == DT_F32)
+    embedding_to_kernel<float, float><<<g, 256, 0, stream>>>(ids, (const float*)table, (float*)out, vocab, width, scale, src, last);
+  else
+    return ERR_BAD_DTYPE;
+  return launch_status();
+}
+
+// out[t, i] = act(in[t, i]) for i < n (in place allowed). act: 0 silu, 1 relu squared, 2 gelu (tanh form).
+extern "C" int dinfer_act(int dtype, int act, const void* in, int64_t ld_in, void* out, int64_t ld_out, int64_t tokens,
+                          int64_t n, hipStream_t stream) {
+  if (tokens <= 0 || n <= 0) return OK;
+  if (act < 0 || act > 2) return ERR_UNSUPPORTED;
+  if (ld_in < n || ld_out < n) return ERR_BAD_SHAPE;
+  for (int64_t t0 = 0; t0 < tokens; t0 += 65535) {
+    const int64_t nt = tokens - t0 < 65535 ? tokens - t0 : 65535;
+    const dim3 grid((unsigned)((n + 1023) / 1024 < 64 ? (n + 1023) / 1024 : 64), (unsigned)nt);
+    DINFER_DISPATCH_DTYPE(dtype, {
+      act_kernel<S><<<grid, 256, 0, stream>>>((const S*)in + t0 * ld_in, ld_in, (S*)out + t0 * ld_out, ld_out, n, act);
+    });
+  }
   return launch_status();
 }

@@ -1,0 +1,408 @@
+// Many small matrix products in one launch, C_g = A_g . W_g^T, and what a routed feed-forward needs around them.
+//
+// Two ways of naming the groups:
+//   heads    group z is a head: A_z, W_z and C_z are column blocks / slabs at fixed strides (a_zs, w_zs, c_zs) and all
+//            groups have the same M rows. With `gate`, row m of C_z is multiplied by sigmoid(gate[m, z]).
+//   experts  group g is an expert: its rows are the entries offsets[g] .. offsets[g+1] of a list sorted by expert
+//            (`perm`: sorted place -> entry = token * top + choice). A row is read either from the entry's token
+//            (a_div = top: the gate and up projections read the step's rows) or from the sorted place itself
+//            (a_div = 0: the down projection reads what the first product left), and written to the sorted place
+//            or, with c_to_perm, to the entry. The work list `tiles` names (expert, first sorted place) of every
+//            row tile; entries beyond the step's tiles hold -1 and their workgroups leave at once.
+// GATED: W_g = [gate rows; up rows] stacked, gate_n rows each, and C = silu(A Wgate^T) * (A Wup^T).
+//
+// Float operands run on the vector ALUs, every output element summed over k in ascending order by one thread (the
+// true 32-bit path; a row's result does not depend on which tile or group size it met). bf16 operands run on the
+// matrix cores: a workgroup of four waves takes 64 x 64 outputs, each wave a 16-row strip, operands read straight
+// from memory in the MFMA's own order (8 consecutive k a lane), float accumulation over ascending k.
+//
+//   moe_route    router logits in float, the `top` largest (lowest index first among equals), softmax over the chosen,
+//                and the shared expert's sigmoid gate
+//   moe_scatter  counts, offsets, the sorted list and the work list, one workgroup (LDS counters)
+//   moe_combine  out[t] = sum_c share[t, c] * y[t * top + c] + shared_gate[t] * shared[t]
+#include "common.cuh"
+
+using namespace dinfer;
+
+namespace {
+
+struct Groups {
+  const void* A; int64_t lda, a_zs;
+  const void* W; int64_t ldw, w_zs;
+  void* C; int64_t ldc, c_zs;
+  int M, N, K;
+  const int32_t* tiles;     // experts: [max_tiles][2]
+  const int32_t* offsets;   // experts: [G + 1]
+  const int32_t* perm;      // experts: sorted place -> entry
+  int a_div;                // experts: > 0: A row = perm[i] / a_div; 0: A row = i
+  int c_to_perm;            // experts: C row = perm[i] instead of i
+  const void* gate; int64_t ld_gate;   // heads: optional
+  int gate_n;               // GATED: rows of each half of W_g
+};
+
+__device__ __forceinline__ float silu(float x) { return x / (1.f + expf(-x)); }
+__device__ __forceinline__ float sigmoid(float x) { return 1.f / (1.f + expf(-x)); }
+
+constexpr int BM = 64, BN = 64, BK = 16;
+
+// Which rows this workgroup's tile holds: group z, local rows [m0, m0 + rows), and for local row r the rows of A and C.
+struct Tile {
+  int z, m0, rows;
+  const int32_t* perm; int a_div, c_to_perm, base;
+  __device__ __forceinline__ bool init(const Groups& p) {
+    if (p.tiles) {
+      z = p.tiles[2 * blockIdx.y];
+      if (z < 0) return false;
+      base = p.tiles[2 * blockIdx.y + 1];
+      m0 = 0;
+      const int end = p.offsets[z + 1];
+      rows = end - base < BM ? end - base : BM;
+      perm = p.perm; a_div = p.a_div; c_to_perm = p.c_to_perm;
+    } else {
+      z = blockIdx.z;
+      m0 = blockIdx.y * BM;
+      rows = p.M - m0 < BM ? p.M - m0 : BM;
+      perm = nullptr; a_div = 0; c_to_perm = 0; base = m0;
+    }
+    return rows > 0;
+  }
+  __device__ __forceinline__ int64_t a_row(int r) const { return perm && a_div > 0 ? perm[base + r] / a_div : base + r; }
+  __device__ __forceinline__ int64_t c_row(int r) const { return perm && c_to_perm ? perm[base + r] : base + r; }
+};
+
+template <class S, class O, bool GATED>
+__global__ void __launch_bounds__(256) grouped_valu_kernel(Groups p) {
+  __shared__ float As[BK][BM + 4];
+  __shared__ float Ws[BK][BN + 4];
+  __shared__ float Us[GATED ? BK : 1][BN + 4];
+  __shared__ int64_t arow[BM];
+  Tile tl;
+  if (!tl.init(p)) return;
+  const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
+  const int n0 = blockIdx.x * BN;
+  const bool experts = p.tiles != nullptr;
+  const S* A = (const S*)p.A + (experts ? 0 : (int64_t)tl.z * p.a_zs);
+  const S* W = (const S*)p.W + (int64_t)tl.z * p.w_zs;
+  if (threadIdx.x < BM) arow[threadIdx.x] = threadIdx.x < tl.rows ? tl.a_row(threadIdx.x) : -1;
+  __syncthreads();
+  float acc[4][4], acu[GATED ? 4 : 1][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      acc[i][j] = 0.f;
+      if (GATED) acu[i][j] = 0.f;
+    }
+  for (int k0 = 0; k0 < p.K; k0 += BK) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int idx = e * 256 + threadIdx.x;
+      const int r = idx >> 4, kk = idx & 15;
+      const int gk = k0 + kk, gn = n0 + r;
+      const int64_t ar = arow[r];
+      As[kk][r] = (ar >= 0 && gk < p.K) ? to_f32(A[ar * p.lda + gk]) : 0.f;
+      Ws[kk][r] = (gn < p.N && gk < p.K) ? to_f32(W[(int64_t)gn * p.ldw + gk]) : 0.f;
+      if (GATED) Us[kk][r] = (gn < p.N && gk < p.K) ? to_f32(W[(int64_t)(gn + p.gate_n) * p.ldw + gk]) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < BK; ++kk) {
+      float a[4], w[4], u[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) a[i] = As[kk][ty * 4 + i];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        w[j] = Ws[kk][tx * 4 + j];
+        if (GATED) u[j] = Us[kk][tx * 4 + j];
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          acc[i][j] = fmaf(a[i], w[j], acc[i][j]);
+          if (GATED) acu[i][j] = fmaf(a[i], u[j], acu[i][j]);
+        }
+    }
+    __syncthreads();
+  }
+  O* C = (O*)p.C + (experts ? 0 : (int64_t)tl.z * p.c_zs);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = ty * 4 + i;
+    if (r >= tl.rows) continue;
+    const int64_t cr = tl.c_row(r);
+    float g = 1.f;
+    if (p.gate) g = sigmoid(to_f32(((const S*)p.gate)[cr * p.ld_gate + tl.z]));
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int gn = n0 + tx * 4 + j;
+      if (gn < p.N) {
+        float v = GATED ? silu(acc[i][j]) * acu[i][j] : acc[i][j];
+        C[cr * p.ldc + gn] = from_f32<O>(v * g);
+      }
+    }
+  }
+}
+
+// bf16 on the matrix cores. A wave owns rows [16 w, 16 w + 16) of the tile and all 64 columns (four 16 x 16 outputs,
+// twice that when gated). v_mfma_f32_16x16x32_bf16: lane l holds row (or column) l % 16 and the 8 consecutive k
+// starting at 8 (l / 16); of the result it holds column l % 16, rows 4 (l / 16) .. + 3.
+template <class O, bool GATED>
+__global__ void __launch_bounds__(256) grouped_mfma_kernel(Groups p) {
+  __shared__ int64_t arow[BM];
+  Tile tl;
+  if (!tl.init(p)) return;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int n0 = blockIdx.x * BN;
+  const bool experts = p.tiles != nullptr;
+  const bf16* A = (const bf16*)p.A + (experts ? 0 : (int64_t)tl.z * p.a_zs);
+  const bf16* W = (const bf16*)p.W + (int64_t)tl.z * p.w_zs;
+  if (threadIdx.x < BM) arow[threadIdx.x] = threadIdx.x < tl.rows ? tl.a_row(threadIdx.x) : -1;
+  __syncthreads();
+  if (wave * 16 >= tl.rows) return;   // (no barrier follows)
+  const int lr = lane & 15, kq = lane >> 4;
+  const int64_t ar = arow[wave * 16 + lr];
+  const bf16* ap = ar >= 0 ? A + ar * p.lda + kq * 8 : nullptr;
+  const bf16* wp[4];
+  const bf16* up[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int gn = n0 + j * 16 + lr;
+    wp[j] = gn < p.N ? W + (int64_t)gn * p.ldw + kq * 8 : nullptr;
+    up[j] = (GATED && gn < p.N) ? W + (int64_t)(gn + p.gate_n) * p.ldw + kq * 8 : nullptr;
+  }
+  bf16x8 zero;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) zero[i] = (bf16)0.f;
+  f32x4 acc[4], acu[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+    acu[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+  const int K = p.K;   // a multiple of 8 (checked on the host)
+  for (int k0 = 0; k0 < K; k0 += 32) {
+    const bool in = k0 + kq * 8 < K;
+    const bf16x8 a = (ap && in) ? *(const bf16x8*)(ap + k0) : zero;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const bf16x8 w = (wp[j] && in) ? *(const bf16x8*)(wp[j] + k0) : zero;
+      acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, w, acc[j], 0, 0, 0);
+      if (GATED) {
+        const bf16x8 u = (up[j] && in) ? *(const bf16x8*)(up[j] + k0) : zero;
+        acu[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, u, acu[j], 0, 0, 0);
+      }
+    }
+  }
+  O* C = (O*)p.C + (experts ? 0 : (int64_t)tl.z * p.c_zs);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = wave * 16 + kq * 4 + i;
+    if (r >= tl.rows) continue;
+    const int64_t cr = tl.c_row(r);
+    float g = 1.f;
+    if (p.gate) g = sigmoid((float)((const bf16*)p.gate)[cr * p.ld_gate + tl.z]);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int gn = n0 + j * 16 + lr;
+      if (gn < p.N) {
+        const float v = GATED ? silu(acc[j][i]) * acu[j][i] : acc[j][i];
+        C[cr * p.ldc + gn] = from_f32<O>(v * g);
+      }
+    }
+  }
+}
+
+// ---- routing ---------------------------------------------------------------------------------------------------
+constexpr int MAX_EXPERTS = 1024;
+
+template <class S>
+__global__ void __launch_bounds__(256) moe_route_kernel(const S* __restrict__ x, int64_t ld_x, const float* __restrict__ wr,
+                                                        const float* __restrict__ wsg, int E, int top, int width,
+                                                        int32_t* __restrict__ idx, float* __restrict__ share,
+                                                        float* __restrict__ shared_gate) {
+  __shared__ float z[MAX_EXPERTS];
+  const int64_t t = blockIdx.x;
+  const S* xr = x + t * ld_x;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  for (int e = wave; e < E + (wsg ? 1 : 0); e += 4) {
+    const float* w = e < E ? wr + (int64_t)e * width : wsg;
+    float acc = 0.f;
+    for (int i = lane; i < width; i += 64) acc = fmaf(to_f32(xr[i]), w[i], acc);
+    acc = wave_sum(acc);
+    if (lane == 0) {
+      if (e < E) z[e] = acc; else shared_gate[t] = sigmoid(acc);
+    }
+  }
+  __syncthreads();
+  if (wave != 0) return;
+  // the `top` largest, one after the other; among equals the lowest index
+  float chosen = 0.f, zmax = 0.f, sum = 0.f;   // lane c keeps the c-th choice
+  int chosen_e = 0;
+  for (int c = 0; c < top; ++c) {
+    float best = -INFINITY;
+    int be = 0x7fffffff;
+    for (int e = lane; e < E; e += 64) {
+      const float v = z[e];
+      if (v > best || (v == best && e < be)) { best = v; be = e; }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      const float ov = __shfl_xor(best, o, 64);
+      const int oe = __shfl_xor(be, o, 64);
+      if (ov > best || (ov == best && oe < be)) { best = ov; be = oe; }
+    }
+    if (c == 0) zmax = best;
+    if (lane == (c & 63)) { chosen = best; chosen_e = be; }
+    if (lane == 0 && be < E) z[be] = -INFINITY;
+    __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    sum += expf(best - zmax);   // every lane holds the same sum, added in the order of the choices
+  }
+  if (lane < top) {
+    idx[t * top + lane] = chosen_e;
+    share[t * top + lane] = expf(chosen - zmax) / sum;
+  }
+}
+
+// One workgroup. entries = tokens * top.
+__global__ void __launch_bounds__(1024) moe_scatter_kernel(const int32_t* __restrict__ idx, int entries, int E, int tile_rows,
+                                                           int32_t* __restrict__ offsets, int32_t* __restrict__ perm,
+                                                           int32_t* __restrict__ tiles, int max_tiles) {
+  __shared__ int cnt[MAX_EXPERTS], off[MAX_EXPERTS + 1], tbase[MAX_EXPERTS + 1];
+  for (int e = threadIdx.x; e < E; e += blockDim.x) cnt[e] = 0;
+  __syncthreads();
+  for (int i = threadIdx.x; i < entries; i += blockDim.x) atomicAdd(&cnt[idx[i]], 1);
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int o = 0, tb = 0;
+    for (int e = 0; e < E; ++e) {
+      off[e] = o; tbase[e] = tb;
+      o += cnt[e];
+      tb += (cnt[e] + tile_rows - 1) / tile_rows;
+    }
+    off[E] = o; tbase[E] = tb;
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e <= E; e += blockDim.x) offsets[e] = off[e];
+  for (int e = threadIdx.x; e < E; e += blockDim.x) {
+    const int n = tbase[e + 1] - tbase[e];
+    for (int k = 0; k < n; ++k) {
+      const int at = tbase[e] + k;
+      if (at < max_tiles) { tiles[2 * at] = e; tiles[2 * at + 1] = off[e] + k * tile_rows; }
+    }
+    cnt[e] = 0;   // now the cursor
+  }
+  for (int at = tbase[E] + threadIdx.x; at < max_tiles; at += blockDim.x) { tiles[2 * at] = -1; tiles[2 * at + 1] = 0; }
+  __syncthreads();
+  for (int i = threadIdx.x; i < entries; i += blockDim.x) {
+    const int e = idx[i];
+    perm[off[e] + atomicAdd(&cnt[e], 1)] = i;
+  }
+}
+
+template <class S>
+__global__ void __launch_bounds__(256) moe_combine_kernel(const S* __restrict__ y, int64_t ld_y, const float* __restrict__ share,
+                                                          int top, const S* __restrict__ shared, int64_t ld_s,
+                                                          const float* __restrict__ shared_gate, S* __restrict__ out,
+                                                          int64_t ld_o, int width) {
+  const int64_t t = blockIdx.x;
+  const float sg = shared ? shared_gate[t] : 0.f;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) {
+    float acc = 0.f;
+    for (int c = 0; c < top; ++c) acc = fmaf(share[t * top + c], to_f32(y[(t * top + c) * ld_y + i]), acc);
+    if (shared) acc = fmaf(sg, to_f32(shared[t * ld_s + i]), acc);
+    out[t * ld_o + i] = from_f32<S>(acc);
+  }
+}
+
+template <bool GATED>
+int launch_groups(int dtype, int out_f32, const Groups& p, dim3 grid, hipStream_t stream) {
+  if (dtype == DT_F32) {
+    grouped_valu_kernel<float, float, GATED><<<grid, 256, 0, stream>>>(p);
+  } else if (dtype == DT_BF16) {
+    const bool mfma = p.K % 8 == 0 && p.lda % 8 == 0 && p.ldw % 8 == 0 && p.a_zs % 8 == 0 && p.w_zs % 8 == 0 &&
+                      ((uintptr_t)p.A % 16) == 0 && ((uintptr_t)p.W % 16) == 0;
+    if (mfma) {
+      if (out_f32) grouped_mfma_kernel<float, GATED><<<grid, 256, 0, stream>>>(p);
+      else grouped_mfma_kernel<bf16, GATED><<<grid, 256, 0, stream>>>(p);
+    } else {
+      if (out_f32) grouped_valu_kernel<bf16, float, GATED><<<grid, 256, 0, stream>>>(p);
+      else grouped_valu_kernel<bf16, bf16, GATED><<<grid, 256, 0, stream>>>(p);
+    }
+  } else {
+    return ERR_BAD_DTYPE;
+  }
+  return launch_status();
+}
+
+}  // namespace
+
+// C[m, z*c_zs + n] = (sigmoid(gate[m, z]) *) sum_k A[m, z*a_zs + k] W[z*w_zs + n*ldw + k], z < groups.
+extern "C" int dinfer_heads_nt(int dtype, const void* A, int64_t lda, int64_t a_zs, const void* W, int64_t ldw,
+                               int64_t w_zs, void* C, int64_t ldc, int64_t c_zs, int64_t M, int64_t N, int64_t K,
+                               int64_t groups, const void* gate, int64_t ld_gate, hipStream_t stream) {
+  if (M <= 0 || N <= 0 || groups <= 0) return OK;
+  if (K <= 0 || ldw < K || M > 0x7fffffff || N > 0x7fffffff || K > 0x7fffffff || groups > 65535) return ERR_BAD_SHAPE;
+  const int64_t gy = (M + BM - 1) / BM;
+  if (gy > 65535) return ERR_UNSUPPORTED;
+  Groups p{};
+  p.A = A; p.lda = lda; p.a_zs = a_zs; p.W = W; p.ldw = ldw; p.w_zs = w_zs; p.C = C; p.ldc = ldc; p.c_zs = c_zs;
+  p.M = (int)M; p.N = (int)N; p.K = (int)K; p.gate = gate; p.ld_gate = ld_gate;
+  const dim3 grid((unsigned)((N + BN - 1) / BN), (unsigned)gy, (unsigned)groups);
+  return launch_groups<false>(dtype, 0, p, grid, stream);
+}
+
+// The products of the experts (see the head of the file). W [experts][rows][ldw] with w_zs elements an expert;
+// gated != 0: rows = 2 N (gate rows, then up rows). max_tiles: the length of `tiles`.
+extern "C" int dinfer_experts_nt(int dtype, int gated, const void* A, int64_t lda, const void* W, int64_t ldw,
+                                 int64_t w_zs, void* C, int64_t ldc, int64_t N, int64_t K, const int32_t* tiles,
+                                 int64_t max_tiles, const int32_t* offsets, const int32_t* perm, int a_div,
+                                 int c_to_perm, hipStream_t stream) {
+  if (N <= 0 || max_tiles <= 0) return OK;
+  if (K <= 0 || ldw < K || lda < K || ldc < N || N > 0x7fffffff || K > 0x7fffffff || max_tiles > 65535 || !tiles ||
+      !offsets || !perm)
+    return ERR_BAD_SHAPE;
+  Groups p{};
+  p.A = A; p.lda = lda; p.W = W; p.ldw = ldw; p.w_zs = w_zs; p.C = C; p.ldc = ldc;
+  p.N = (int)N; p.K = (int)K; p.tiles = tiles; p.offsets = offsets; p.perm = perm; p.a_div = a_div;
+  p.c_to_perm = c_to_perm; p.gate_n = (int)N;
+  const dim3 grid((unsigned)((N + BN - 1) / BN), (unsigned)max_tiles, 1);
+  return gated ? launch_groups<true>(dtype, 0, p, grid, stream) : launch_groups<false>(dtype, 0, p, grid, stream);
+}
+
+extern "C" int dinfer_moe_tile_rows() { return BM; }
+
+extern "C" int dinfer_moe_route(int dtype, const void* x, int64_t ld_x, int64_t tokens, const float* router,
+                                const float* shared_gate_w, int experts, int top, int width, int32_t* idx, float* share,
+                                float* shared_gate, hipStream_t stream) {
+  if (tokens <= 0) return OK;
+  if (experts <= 0 || top <= 0 || top > experts || width <= 0 || tokens > 0x7fffffff) return ERR_BAD_SHAPE;
+  if (experts > MAX_EXPERTS || top > 64) return ERR_UNSUPPORTED;
+  DINFER_DISPATCH_DTYPE(dtype, {
+    moe_route_kernel<S><<<(unsigned)tokens, 256, 0, stream>>>((const S*)x, ld_x, router, shared_gate_w, experts, top,
+                                                             width, idx, share, shared_gate);
+  });
+  return launch_status();
+}
+
+extern "C" int dinfer_moe_scatter(const int32_t* idx, int64_t entries, int experts, int32_t* offsets, int32_t* perm,
+                                  int32_t* tiles, int64_t max_tiles, hipStream_t stream) {
+  if (entries <= 0) return OK;
+  if (experts <= 0 || entries > 0x7fffffff || max_tiles < (entries + BM - 1) / BM + experts) return ERR_BAD_SHAPE;
+  if (experts > MAX_EXPERTS) return ERR_UNSUPPORTED;
+  moe_scatter_kernel<<<1, 1024, 0, stream>>>(idx, (int)entries, experts, BM, offsets, perm, tiles, (int)max_tiles);
+  return launch_status();
+}
+
+extern "C" int dinfer_moe_combine(int dtype, const void* y, int64_t ld_y, const float* share, int top, const void* shared,
+                                  int64_t ld_s, const float* shared_gate, void* out, int64_t ld_o, int64_t tokens,
+                                  int width, hipStream_t stream) {
+  if (tokens <= 0) return OK;
+  if (top <= 0 || width <= 0 || tokens > 0x7fffffff) return ERR_BAD_SHAPE;
+  DINFER_DISPATCH_DTYPE(dtype, {
+    moe_combine_kernel<S><<<(unsigned)tokens, 256, 0, stream>>>((const S*)y, ld_y, share, top, (const S*)shared, ld_s,
+                                                               shared_gate, (S*)out, ld_o, width);
+  });
+  return launch_status();
+}

@@ -108,6 +108,50 @@ __global__ void __launch_bounds__(256) rmsnorm_bf16x8_kernel(const bf16* __restr
   }
 }
 
+// Layer norm with gain and bias over the last dimension: y = (x - mean) / sqrt(var + eps) * w + b, var the mean of the
+// squared deviations (two passes over the row, which waits in LDS in float). The operands may differ in storage: the
+// residual stream may be float where the branch added to it and the normed row are bf16. With a residual,
+// r = round(x + r) is written back in the residual's own type first and normed as stored.
+__device__ __forceinline__ float ld_any(const void* p, int64_t i, int dt) {
+  return dt == DT_F32 ? ((const float*)p)[i] : (float)((const bf16*)p)[i];
+}
+__device__ __forceinline__ void st_any(void* p, int64_t i, int dt, float v) {
+  if (dt == DT_F32) ((float*)p)[i] = v; else ((bf16*)p)[i] = (bf16)v;
+}
+__device__ __forceinline__ float round_any(float v, int dt) { return dt == DT_F32 ? v : (float)(bf16)v; }
+
+__global__ void __launch_bounds__(256) layernorm_kernel(const void* __restrict__ x, int x_dt, void* __restrict__ residual,
+                                                        int r_dt, const int32_t* __restrict__ rows,
+                                                        const void* __restrict__ w, const void* __restrict__ b, int p_dt,
+                                                        void* __restrict__ out, int o_dt, int64_t width, int64_t ld_x,
+                                                        int64_t ld_res, float eps) {
+  extern __shared__ float row[];
+  __shared__ float red[16];
+  const int64_t r = blockIdx.x;
+  const int64_t src = rows ? (int64_t)rows[r] : r;
+  float sum = 0.f;
+  for (int64_t i = threadIdx.x; i < width; i += blockDim.x) {
+    float v = ld_any(x, src * ld_x + i, x_dt);
+    if (residual) {
+      v = round_any(v + ld_any(residual, src * ld_res + i, r_dt), r_dt);
+      st_any(residual, src * ld_res + i, r_dt, v);
+    }
+    row[i] = v;
+    sum += v;
+  }
+  const float mean = block_sum(sum, red) / (float)width;
+  float ss = 0.f;
+  for (int64_t i = threadIdx.x; i < width; i += blockDim.x) {   // each thread re-reads what it wrote itself
+    const float d = row[i] - mean;
+    ss = add_square(ss, d);
+  }
+  const float inv = 1.f / sqrtf(block_sum(ss, red) / (float)width + eps);
+  for (int64_t i = threadIdx.x; i < width; i += blockDim.x) {
+    const float y = (row[i] - mean) * inv * ld_any(w, i, p_dt) + (b ? ld_any(b, i, p_dt) : 0.f);
+    st_any(out, r * width + i, o_dt, y);
+  }
+}
+
 inline bool aligned16(const void* p) { return ((uintptr_t)p % 16) == 0; }
 
 }  // namespace
@@ -145,5 +189,20 @@ extern "C" int dinfer_rmsnorm(int dtype, const void* x, void* residual, const in
   } else {
     return ERR_BAD_DTYPE;
   }
+  return launch_status();
+}
+
+// x, residual (may be null), w and b (b may be null) and out each with a dtype code of their own (w and b share one).
+// out is dense [n_rows, width]. Width up to 16,384 (the row waits in LDS).
+extern "C" int dinfer_layernorm(const void* x, int x_dtype, void* residual, int res_dtype, const int32_t* rows,
+                                const void* w, const void* b, int param_dtype, void* out, int out_dtype, int64_t n_rows,
+                                int64_t width, int64_t ld_x, int64_t ld_res, float eps, hipStream_t stream) {
+  if (n_rows <= 0) return OK;
+  if (width <= 0 || ld_x < width || (residual && ld_res < width) || n_rows > 0x7fffffff) return ERR_BAD_SHAPE;
+  for (int dt : {x_dtype, res_dtype, param_dtype, out_dtype})
+    if (dt != DT_F32 && dt != DT_BF16) return ERR_BAD_DTYPE;
+  if (width > 16384) return ERR_UNSUPPORTED;
+  layernorm_kernel<<<(unsigned)n_rows, 256, (size_t)width * sizeof(float), stream>>>(
+      x, x_dtype, residual, res_dtype, rows, w, b, param_dtype, out, out_dtype, width, ld_x, ld_res, eps);
   return launch_status();
 }

@@ -24,6 +24,17 @@ SIGNATURES = {
     "dinfer_scale_softcap": ("elementwise", [_I, _P, _L, _L, _L, _F, _F, _P]),
     "dinfer_widen": ("elementwise", [_I, _P, _P, _L, _P]),
     "dinfer_fill_u32": ("elementwise", [_P, c_uint32, _L, _P]),
+    "dinfer_embedding_to": ("elementwise", [_I, _I, _P, _P, _P, _L, _L, _L, _F, _P, _P, _P]),
+    "dinfer_act": ("elementwise", [_I, _I, _P, _L, _P, _L, _L, _L, _P]),
+    "dinfer_layernorm": ("norm", [_P, _I, _P, _I, _P, _P, _P, _I, _P, _I, _L, _L, _L, _L, _F, _P]),
+    "dinfer_latent_post": ("latent", [_I, _P, _L, _L, _I, _I, _I, _I, _I, _I, _P, _I, _F, _P, _P, _I, _P, _L, _P, _P, _P]),
+    "dinfer_latent_attn_ref": ("latent", [_I, _P, _L, _P, _L, _P, _P, _L, _P, _P, _I, _L, _F, _I, _I, _I, _I, _I, _P]),
+    "dinfer_heads_nt": ("grouped", [_I, _P, _L, _L, _P, _L, _L, _P, _L, _L, _L, _L, _L, _L, _P, _L, _P]),
+    "dinfer_experts_nt": ("grouped", [_I, _I, _P, _L, _P, _L, _L, _P, _L, _L, _L, _P, _L, _P, _P, _I, _I, _P]),
+    "dinfer_moe_tile_rows": ("grouped", []),
+    "dinfer_moe_route": ("grouped", [_I, _P, _L, _L, _P, _P, _I, _I, _I, _P, _P, _P, _P]),
+    "dinfer_moe_scatter": ("grouped", [_P, _L, _I, _P, _P, _P, _L, _P]),
+    "dinfer_moe_combine": ("grouped", [_I, _P, _L, _P, _I, _P, _L, _P, _P, _L, _L, _I, _P]),
     "dinfer_rmsnorm": ("norm", [_I, _P, _P, _P, _P, _I, _P, _L, _L, _L, _L, _F, _F, _P]),
     "dinfer_qkv_post": (
         "rope",

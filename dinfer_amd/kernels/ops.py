@@ -60,18 +60,22 @@ def _is_param_f32(w: torch.Tensor, act_dtype: torch.dtype) -> int:
 
 
 def embedding(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor, src: torch.Tensor | None = None,
-              last: torch.Tensor | None = None) -> torch.Tensor:
-    """out[t] = table[ids[t]]; ids int32 [T], table [V, W], out [T, W]. src, last (int32, both or neither): where
+              last: torch.Tensor | None = None, scale: float = 1.0) -> torch.Tensor:
+    """out[t] = table[ids[t]] * scale; ids int32 [T], table [V, W], out [T, W] (out may be float32 beside a bfloat16 table). src, last (int32, both or neither): where
     src[t] >= 0 the id is last[src[t]], a token the step before sampled, which only the device knows so far."""
     _need_gpu(ids, table, out, src, last)
     assert ids.dtype == torch.int32 and ids.is_contiguous()
     assert (src is None) == (last is None)
     if src is not None:
         assert src.dtype == last.dtype == torch.int32 and src.numel() >= ids.numel()
-    assert table.is_contiguous() and out.is_contiguous() and table.dtype == out.dtype
+    assert table.is_contiguous() and out.is_contiguous()
     T = ids.numel()
     V, W = table.shape
     assert out.shape[0] >= T and out.shape[1] == W
+    if scale != 1.0 or table.dtype != out.dtype:     # a stream wider than the table, or a multiplied embedding
+        lib.call("dinfer_embedding_to", dtype_code(table.dtype), dtype_code(out.dtype), ids.data_ptr(), table.data_ptr(),
+                 out.data_ptr(), T, V, W, float(scale), _ptr(src), _ptr(last), _stream())
+        return out
     lib.call("dinfer_embedding", dtype_code(table.dtype), ids.data_ptr(), table.data_ptr(), out.data_ptr(), T, V, W,
              _ptr(src), _ptr(last), _stream())
     return out
@@ -147,6 +151,203 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor, eps: float
     lib.call("dinfer_rmsnorm", dtype_code(x.dtype), x.data_ptr(), _ptr(residual), _ptr(rows), weight.data_ptr(),
              _is_param_f32(weight, x.dtype), out.data_ptr(), n_rows, width, _rows(x),
              _rows(residual) if residual is not None else 0, float(eps), float(weight_offset), _stream())
+    return out
+
+
+ACTS = {"silu": 0, "relu2": 1, "gelu_tanh": 2}   # activations of one argument -> their code in the C interface
+
+
+def act(x: torch.Tensor, out: torch.Tensor, tokens: int, kind: str) -> torch.Tensor:
+    """out[t, i] = act(x[t, i]); out may be x."""
+    _need_gpu(x, out)
+    if kind not in ACTS:
+        raise lib.KernelError(f"activation {kind!r} has no kernel (known: {sorted(ACTS)})")
+    n = out.shape[1]
+    assert x.shape[1] == n and x.dtype == out.dtype and x.shape[0] >= tokens and out.shape[0] >= tokens
+    lib.call("dinfer_act", dtype_code(x.dtype), ACTS[kind], x.data_ptr(), _rows(x), out.data_ptr(), _rows(out), tokens, n,
+             _stream())
+    return out
+
+
+def layernorm(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, out: torch.Tensor, eps: float,
+              n_rows: int, *, residual: torch.Tensor | None = None, rows: torch.Tensor | None = None) -> torch.Tensor:
+    """out[r] = (x[src r] - mean) / sqrt(var + eps) * weight + bias, in float. residual: updated in place to
+    round(x + residual) in its own type first (it may be float32 beside a bfloat16 x), and that sum is normed.
+    rows: int32 indices of the n_rows source rows; default identity."""
+    _need_gpu(x, weight, bias, out, residual, rows)
+    width = out.shape[1]
+    assert x.shape[1] == width and weight.numel() == width and weight.is_contiguous() and out.is_contiguous()
+    assert bias is None or (bias.numel() == width and bias.is_contiguous() and bias.dtype == weight.dtype)
+    assert out.shape[0] >= n_rows
+    if rows is None:
+        assert x.shape[0] >= n_rows
+    else:
+        assert rows.dtype == torch.int32 and rows.is_contiguous() and rows.numel() >= n_rows
+    if residual is not None:
+        assert residual.shape == x.shape
+    lib.call("dinfer_layernorm", x.data_ptr(), dtype_code(x.dtype), _ptr(residual),
+             dtype_code(residual.dtype) if residual is not None else 0, _ptr(rows), weight.data_ptr(), _ptr(bias),
+             dtype_code(weight.dtype), out.data_ptr(), dtype_code(out.dtype), n_rows, width, _rows(x),
+             _rows(residual) if residual is not None else 0, float(eps), _stream())
+    return out
+
+
+# ---- latent attention ----------------------------------------------------------------------------
+# Cache pages [blocks, page, R + dr]: one row a token, the normed latent and then the rotated shared key part.
+LATENT_MAX_RANK = 1024   # the largest latent the attention kernels hold in registers
+LATENT_MAX_KEY = 1280    # the largest latent + rotated part
+
+
+def latent_cache_shape(blocks: int, page_size: int, rank: int, rot_dim: int) -> tuple:
+    return (blocks, page_size, rank + rot_dim)
+
+
+def latent_post(proj: torch.Tensor, tokens: int, *, heads: int, dim: int, rot_dim: int, rank: int, q_off: int,
+                c_off: int | None, gain: torch.Tensor | None, eps: float, positions: torch.Tensor,
+                cos_sin: torch.Tensor | None, rotary_dim: int, qa: torch.Tensor, cache: torch.Tensor | None,
+                slot_mapping: torch.Tensor | None) -> None:
+    """From the step's projections: every head's rotated query part goes, rotated, into qa (head h at h*(rank+rot_dim),
+    behind the rank entries the caller fills), and, where the layer has a down projection of its own (c_off), the
+    token's latent (RMS-normed with `gain`) and rotated shared key part go to its cache slot."""
+    _need_gpu(proj, gain, positions, cos_sin, qa, cache, slot_mapping)
+    assert proj.shape[0] >= tokens and qa.shape[0] >= tokens and qa.dtype == proj.dtype
+    assert q_off + heads * (dim + rot_dim) <= proj.shape[1] and qa.shape[1] >= heads * (rank + rot_dim)
+    assert positions.dtype == torch.int32 and positions.numel() >= tokens
+    if cos_sin is not None:
+        assert cos_sin.dtype == torch.float32 and cos_sin.is_contiguous() and cos_sin.shape[1] == rotary_dim
+    write = c_off is not None and slot_mapping is not None
+    if write:
+        assert c_off + rank + rot_dim <= proj.shape[1] and gain is not None and gain.numel() == rank
+        assert slot_mapping.dtype == torch.int64 and slot_mapping.numel() >= tokens
+        assert cache is not None and cache.dtype == proj.dtype and cache.is_contiguous()
+        assert cache.shape[-1] == rank + rot_dim
+    lib.call("dinfer_latent_post", dtype_code(proj.dtype), proj.data_ptr(), tokens, _rows(proj), q_off,
+             c_off if write else -1, heads, dim, rot_dim, rank, _ptr(gain) if write else 0,
+             _is_param_f32(gain, proj.dtype) if write else 0, float(eps), positions.data_ptr(), _ptr(cos_sin),
+             rotary_dim if cos_sin is not None else 0, qa.data_ptr(), _rows(qa), _ptr(cache) if write else 0,
+             _ptr(slot_mapping) if write else 0, _stream())
+
+
+def _check_latent(qa, out, cache, block_table, cu_seqlens, seq_lens, num_reqs, tokens, heads, rank, rot_dim, page_size):
+    assert qa.dtype == out.dtype == cache.dtype and cache.is_contiguous()
+    assert tuple(cache.shape[1:]) == (page_size, rank + rot_dim)
+    assert block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.is_contiguous()
+    assert block_table.shape[0] >= num_reqs
+    assert cu_seqlens.dtype == torch.int32 and cu_seqlens.numel() >= num_reqs + 1
+    assert seq_lens.dtype == torch.int32 and seq_lens.numel() >= num_reqs
+    assert qa.shape[1] >= heads * (rank + rot_dim) and out.shape[1] >= heads * rank
+    assert qa.shape[0] >= tokens and out.shape[0] >= tokens
+
+
+def latent_attn_ref(qa: torch.Tensor, out: torch.Tensor, cache: torch.Tensor, block_table: torch.Tensor,
+                    cu_seqlens: torch.Tensor, seq_lens: torch.Tensor, num_reqs: int, tokens: int, *, scale: float,
+                    window: int, heads: int, rank: int, rot_dim: int, page_size: int) -> torch.Tensor:
+    """Plain attention over the latent pages (any sizes, float arithmetic): out[t, h*rank : (h+1)*rank] = the
+    softmax-weighted sum of the latents, scores scale * <qa[t, h], cache row>."""
+    _need_gpu(qa, out, cache, block_table, cu_seqlens, seq_lens)
+    _check_latent(qa, out, cache, block_table, cu_seqlens, seq_lens, num_reqs, tokens, heads, rank, rot_dim, page_size)
+    lib.call("dinfer_latent_attn_ref", dtype_code(qa.dtype), qa.data_ptr(), _rows(qa), out.data_ptr(), _rows(out),
+             cache.data_ptr(), block_table.data_ptr(), block_table.shape[1], cu_seqlens.data_ptr(), seq_lens.data_ptr(),
+             num_reqs, tokens, float(scale), int(window), heads, rank, rot_dim, page_size, _stream())
+    return out
+
+
+def latent_mfma_supports(rank: int, rot_dim: int) -> bool:
+    return False
+
+
+# ---- many small products in one launch ---------------------------------------------------------------
+def heads_nt(a: torch.Tensor, a_off: int, a_stride: int, w: torch.Tensor, out: torch.Tensor, c_off: int, c_stride: int,
+             m: int, *, gate: torch.Tensor | None = None, gate_off: int = 0) -> torch.Tensor:
+    """For every head z: out[:m, c_off + z*c_stride : ... + N] = a[:m, a_off + z*a_stride : ... + K] @ w[z].T with
+    w [heads, N, K]; gate: the rows of head z are multiplied by sigmoid(gate[:, gate_off + z])."""
+    _need_gpu(a, w, out, gate)
+    heads, n, k = w.shape
+    assert w.is_contiguous() and a.dtype == w.dtype == out.dtype
+    assert a.shape[0] >= m and out.shape[0] >= m
+    assert a_off + (heads - 1) * a_stride + k <= a.shape[1] and c_off + (heads - 1) * c_stride + n <= out.shape[1]
+    es = a.element_size()
+    if gate is not None:
+        assert gate.dtype == a.dtype and gate.shape[0] >= m and gate_off + heads <= gate.shape[1]
+    lib.call("dinfer_heads_nt", dtype_code(a.dtype), a.data_ptr() + a_off * es, _rows(a), a_stride, w.data_ptr(), k, n * k,
+             out.data_ptr() + c_off * es, _rows(out), c_stride, m, n, k, heads,
+             gate.data_ptr() + gate_off * es if gate is not None else 0, _rows(gate) if gate is not None else 0, _stream())
+    return out
+
+
+MOE_MAX_EXPERTS = 1024   # the routing and sorting kernels keep one number an expert in LDS
+MOE_MAX_TOP = 64         # a lane of the routing wave keeps one choice
+
+
+def moe_tile_rows() -> int:
+    return int(lib.get("dinfer_moe_tile_rows")())
+
+
+def moe_max_tiles(entries: int, experts: int) -> int:
+    """Length of the work list for `entries` (token, choice) pairs: every expert may end with a tile that is not full."""
+    return -(-entries // moe_tile_rows()) + experts
+
+
+def moe_route(x: torch.Tensor, router: torch.Tensor, shared_gate_w: torch.Tensor | None, idx: torch.Tensor,
+              share: torch.Tensor, shared_gate: torch.Tensor | None, tokens: int, top: int) -> None:
+    """Per token: logits x @ router.T in float (router float32 [experts, width]), idx[t] the `top` largest (lowest index
+    among equals), share[t] the softmax over them; shared_gate[t] = sigmoid(x . shared_gate_w) where that is given."""
+    _need_gpu(x, router, shared_gate_w, idx, share, shared_gate)
+    experts, width = router.shape
+    assert router.dtype == torch.float32 and router.is_contiguous() and x.shape[1] == width and x.shape[0] >= tokens
+    assert idx.dtype == torch.int32 and share.dtype == torch.float32 and idx.is_contiguous() and share.is_contiguous()
+    assert idx.numel() >= tokens * top and share.numel() >= tokens * top
+    if shared_gate_w is not None:
+        assert shared_gate_w.dtype == torch.float32 and shared_gate_w.numel() == width and shared_gate_w.is_contiguous()
+        assert shared_gate is not None and shared_gate.dtype == torch.float32 and shared_gate.numel() >= tokens
+    lib.call("dinfer_moe_route", dtype_code(x.dtype), x.data_ptr(), _rows(x), tokens, router.data_ptr(),
+             _ptr(shared_gate_w), experts, top, width, idx.data_ptr(), share.data_ptr(),
+             _ptr(shared_gate) if shared_gate_w is not None else 0, _stream())
+
+
+def moe_scatter(idx: torch.Tensor, entries: int, experts: int, offsets: torch.Tensor, perm: torch.Tensor,
+                tiles: torch.Tensor) -> None:
+    """Sorts the entries (token * top + choice) by expert: offsets [experts + 1], perm [entries] (sorted place -> entry),
+    tiles [n, 2] the work list of experts_nt ((expert, first sorted place) per row tile, -1 beyond the last)."""
+    _need_gpu(idx, offsets, perm, tiles)
+    assert idx.dtype == offsets.dtype == perm.dtype == tiles.dtype == torch.int32
+    assert idx.numel() >= entries and perm.numel() >= entries and offsets.numel() >= experts + 1
+    assert tiles.is_contiguous() and tiles.dim() == 2 and tiles.shape[1] == 2
+    n = moe_max_tiles(entries, experts)
+    assert tiles.shape[0] >= n
+    lib.call("dinfer_moe_scatter", idx.data_ptr(), entries, experts, offsets.data_ptr(), perm.data_ptr(),
+             tiles.data_ptr(), n, _stream())
+
+
+def experts_nt(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, entries: int, tiles: torch.Tensor,
+               offsets: torch.Tensor, perm: torch.Tensor, *, gated: bool, a_div: int, c_to_perm: bool) -> torch.Tensor:
+    """The products of all experts in one launch. w [experts, rows, K]; gated: rows = 2 N, gate rows first, and
+    out = silu(a Wg^T) * (a Wu^T). a_div > 0: the row of sorted place i is a[perm[i] // a_div] (the step's tokens),
+    0: a[i]. c_to_perm: the result of sorted place i goes to out[perm[i]], else to out[i]."""
+    _need_gpu(a, w, out, tiles, offsets, perm)
+    experts, rows, k = w.shape
+    n = rows // 2 if gated else rows
+    assert w.is_contiguous() and a.dtype == w.dtype == out.dtype and a.shape[1] == k and out.shape[1] == n
+    assert out.shape[0] >= entries and (a_div > 0 or a.shape[0] >= entries)
+    lib.call("dinfer_experts_nt", dtype_code(a.dtype), 1 if gated else 0, a.data_ptr(), _rows(a), w.data_ptr(), k,
+             rows * k, out.data_ptr(), _rows(out), n, k, tiles.data_ptr(), moe_max_tiles(entries, experts),
+             offsets.data_ptr(), perm.data_ptr(), int(a_div), 1 if c_to_perm else 0, _stream())
+    return out
+
+
+def moe_combine(y: torch.Tensor, share: torch.Tensor, top: int, shared: torch.Tensor | None,
+                shared_gate: torch.Tensor | None, out: torch.Tensor, tokens: int) -> torch.Tensor:
+    """out[t] = sum_c share[t, c] * y[t * top + c] (+ shared_gate[t] * shared[t])."""
+    _need_gpu(y, share, shared, shared_gate, out)
+    width = out.shape[1]
+    assert y.shape[1] == width and y.dtype == out.dtype and y.shape[0] >= tokens * top and out.shape[0] >= tokens
+    assert share.dtype == torch.float32 and share.numel() >= tokens * top
+    if shared is not None:
+        assert shared.dtype == out.dtype and shared.shape[1] == width and shared.shape[0] >= tokens
+        assert shared_gate is not None and shared_gate.dtype == torch.float32 and shared_gate.numel() >= tokens
+    lib.call("dinfer_moe_combine", dtype_code(y.dtype), y.data_ptr(), _rows(y), share.data_ptr(), top, _ptr(shared),
+             _rows(shared) if shared is not None else 0, _ptr(shared_gate), out.data_ptr(), _rows(out), tokens, width,
+             _stream())
     return out
 
 

@@ -1,1 +1,1 @@
-from . import qwen3  # noqa: F401  (registers Qwen3ForCausalLM)
+from . import kudurax, qwen3  # noqa: F401  (register the built-in architectures)

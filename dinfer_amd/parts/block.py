@@ -43,9 +43,12 @@ class PreNormBlock(Block):
         self.ff = FEED_FORWARDS.get(layer.feed_forward.kind)(hidden=hidden, **layer.feed_forward.params)
         ncls = NORMS.get(layer.norm.kind)
         self.norm_in, self.norm_post = ncls(hidden, **layer.norm.params), ncls(hidden, **layer.norm.params)
+        if getattr(self.ff, "absent", False):      # a layer that is its mixer alone: h += mixer(norm_in(h))
+            self.ff = self.norm_post = None
 
     def _parts(self):
-        return zip(self.prefixes, (self.mixer, self.ff, self.norm_in, self.norm_post))
+        return [(p, part) for p, part in zip(self.prefixes, (self.mixer, self.ff, self.norm_in, self.norm_post))
+                if part is not None]
 
     @property
     def capturable(self):
@@ -88,6 +91,8 @@ class PreNormBlock(Block):
             x = self.norm_in.forward(hidden, self.normed, T)
         else:
             x = self.norm_in.forward(pending, self.normed, T, residual=hidden)
+        if self.ff is None:
+            return self.mixer.forward(x, batch, cache, **self._into(hidden, next_norm, self.mixer, T))
         a = self.mixer.forward(x, batch, cache, **self._into(hidden, self.norm_post, self.mixer, T))
         if isinstance(a, Carried):
             x = a if self.ff.carries_norms else a.materialise()

@@ -126,7 +126,8 @@ class DecoderModel:
             if op is not None:
                 op[1].bind(ctx)
         ws = ctx.workspace
-        self.hidden = ws.buffer("hidden", self.spec.hidden_size)
+        stream = torch.float32 if self.spec.stream_dtype == "float32" else None
+        self.hidden = ws.buffer("hidden", self.spec.hidden_size, dtype=stream)
         self.final_normed = ws.buffer("final_normed", self.spec.hidden_size, rows=ctx.max_rows)
         self.logits = torch.empty((ctx.max_rows, self.spec.vocab_size), dtype=torch.float32, device=ctx.device)
 
@@ -135,7 +136,7 @@ class DecoderModel:
         at batch.logits_rows (a view of a fixed buffer)."""
         T, R = batch.num_tokens, batch.num_rows
         ops.embedding(batch.input_ids[:T], self.embed, self.hidden, getattr(batch, "feedback_src", None),
-                      getattr(batch, "last_tokens", None))
+                      getattr(batch, "last_tokens", None), scale=self.spec.embed_scale)
         if self.embed_post is not None:
             self.embed_post[1].forward(self.hidden, T)
         pending = None

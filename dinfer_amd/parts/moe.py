@@ -1,0 +1,93 @@
+"""Routed feed-forward (mixture of experts).
+
+    z = Wr x  (float)            the `top` experts with the largest z are chosen per token,
+    p = softmax over the chosen z only
+    y = sum_chosen p_e * down_e( silu(gate_e x) * up_e x )
+        + sigmoid(wsg . x) * shared(x)          (a gated feed-forward every token runs, where the layer has one)
+
+Per step: one kernel routes (logits, choice, weights, the shared gate), one sorts the (token, choice) entries by
+expert and writes the work list of row tiles, two launches run the products of all experts (gate and up with the
+activation, then down, each row computed alone and written to its entry's place), and one sums a token's entries in
+the order of its choices. Launch shapes depend on the step's token count alone; which expert gets which rows is read
+from device memory, so the step may be captured. No atomics on results: a token's output does not depend on what
+else is in the batch.
+"""
+from __future__ import annotations
+
+import torch
+
+from ..kernels import ops
+from .base import FeedForward
+from .mlp import GatedMLP
+from .registry import FEED_FORWARDS
+from .spec import TensorSpec
+
+
+@FEED_FORWARDS.register("moe")
+class RoutedExperts(FeedForward):
+    """Tensors: e<i>.gate / .up / .down per expert, router [experts, hidden]; shared.gate / .up / .down and shared.sg
+    [1, hidden] where `shared_intermediate` is given."""
+
+    def __init__(self, hidden: int, experts: int, top: int, intermediate: int, shared_intermediate: int | None = None,
+                 act: str = "silu"):
+        if act != "silu":
+            raise ValueError(f"routed feed-forward: activation {act!r} has no kernel (known: ['silu'])")
+        if not (0 < top <= experts) or experts > ops.MOE_MAX_EXPERTS or top > ops.MOE_MAX_TOP:
+            raise ValueError(f"routed feed-forward: {top} of {experts} experts has no kernel (up to {ops.MOE_MAX_TOP} of "
+                             f"{ops.MOE_MAX_EXPERTS})")
+        self.hidden, self.experts, self.top, self.intermediate = hidden, experts, top, intermediate
+        self.shared = None
+        if shared_intermediate:
+            self.shared = GatedMLP(hidden, shared_intermediate, act, names=("shared.gate", "shared.up", "shared.down"),
+                                   out_name="shared_out")
+
+    def tensors(self):
+        t = {"router": TensorSpec((self.experts, self.hidden))}
+        for e in range(self.experts):
+            t[f"e{e}.gate"] = TensorSpec((self.intermediate, self.hidden))
+            t[f"e{e}.up"] = TensorSpec((self.intermediate, self.hidden))
+            t[f"e{e}.down"] = TensorSpec((self.hidden, self.intermediate))
+        if self.shared is not None:
+            t.update(self.shared.tensors())
+            t["shared.sg"] = TensorSpec((1, self.hidden))
+        return t
+
+    def load(self, get):
+        self.router = get("router").float().contiguous()       # routing runs in 32 bits
+        E = range(self.experts)
+        # [experts, 2 I, hidden]: an expert's gate rows, then its up rows; [experts, hidden, I]
+        self.w_in = torch.stack([torch.cat([get(f"e{e}.gate", compute=True), get(f"e{e}.up", compute=True)], dim=0)
+                                 for e in E]).contiguous()
+        self.w_out = torch.stack([get(f"e{e}.down", compute=True) for e in E]).contiguous()
+        self.sg = None
+        if self.shared is not None:
+            self.shared.load(get)
+            self.sg = get("shared.sg").float().reshape(-1).contiguous()
+
+    def bind(self, ctx):
+        ws, dev = ctx.workspace, ctx.device
+        n = ctx.max_tokens * self.top
+        i32 = torch.int32
+        self.idx = torch.zeros(n, dtype=i32, device=dev)
+        self.share = torch.zeros(n, dtype=torch.float32, device=dev)
+        self.shared_gate = torch.zeros(ctx.max_tokens, dtype=torch.float32, device=dev)
+        self.offsets = torch.zeros(self.experts + 1, dtype=i32, device=dev)
+        self.perm = torch.zeros(n, dtype=i32, device=dev)
+        self.tiles = torch.zeros((ops.moe_max_tiles(n, self.experts), 2), dtype=i32, device=dev)
+        self.act_buf = ws.buffer("moe_act", self.intermediate, rows=n)
+        self.y_buf = ws.buffer("moe_y", self.hidden, rows=n)
+        self.out_buf = ws.buffer("ffn_out", self.hidden)
+        if self.shared is not None:
+            self.shared.bind(ctx)
+
+    def forward(self, x, batch, into=None):
+        T, top = batch.num_tokens, self.top
+        n = T * top
+        ops.moe_route(x, self.router, self.sg, self.idx, self.share, self.shared_gate, T, top)
+        ops.moe_scatter(self.idx, n, self.experts, self.offsets, self.perm, self.tiles)
+        ops.experts_nt(x, self.w_in, self.act_buf, n, self.tiles, self.offsets, self.perm, gated=True, a_div=top,
+                       c_to_perm=False)
+        ops.experts_nt(self.act_buf, self.w_out, self.y_buf, n, self.tiles, self.offsets, self.perm, gated=False, a_div=0,
+                       c_to_perm=True)
+        shared = self.shared.forward(x, batch) if self.shared is not None else None
+        return ops.moe_combine(self.y_buf, self.share, top, shared, self.shared_gate, self.out_buf, T)

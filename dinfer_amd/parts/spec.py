@@ -103,6 +103,27 @@ class KVSpec(CacheSpec):
 
 
 @dataclass(frozen=True)
+class LatentSpec(CacheSpec):
+    """Cache need of a mixer that stores one row a token which all its heads share: `rank` numbers of a latent from
+    which keys and values are made, and `rot_dim` numbers of a rotated key part. Pages [blocks, page, rank + rot_dim]."""
+    rank: int
+    rot_dim: int
+    window: int | None = None
+
+    def group_key(self) -> tuple:
+        return ("latent", self.rank, self.rot_dim, self.window)
+
+    def page_bytes(self, page_size, dtype):
+        return (self.rank + self.rot_dim) * page_size * _element_size(dtype)
+
+    def allocate(self, num_blocks, page_size, num_slots, dtype, device):
+        import torch
+        from ..kernels import ops
+        shape = ops.latent_cache_shape(num_blocks, page_size, self.rank, self.rot_dim)
+        return {"latent": torch.zeros(shape, dtype=dtype, device=device)}
+
+
+@dataclass(frozen=True)
 class StateSpec(CacheSpec):
     """Cache need of a mixer with per-request state of fixed size (shape per request). The state cannot be rebuilt
     from pages, so a model that has one gets no prefix cache."""
@@ -170,3 +191,8 @@ class ModelSpec:
     # its own under embed_name + "post.") and to the logits after the head (under head_name + "post.")
     embed_post: PartSpec | None = None
     logits_post: PartSpec | None = None
+    # the embeddings are multiplied by this on their way into the stream (inside the gather)
+    embed_scale: float = 1.0
+    # "float32": the residual stream is kept in 32 bits whatever the engine's dtype (the blocks' norms read it and write
+    # the engine's dtype); None: the engine's dtype
+    stream_dtype: str | None = None
