@@ -7,17 +7,23 @@
 //   ol_h = sum_j softmax(s)_j c_j                (R numbers a head; the caller multiplies by Wuv_h)
 //
 // which is attention with one shared key/value head whose keys are R + dr wide and whose values are the first R
-// numbers of the same row. Cache pages: [blocks][page][R + dr], one row a token.
+// numbers of the same row. Cache pages: [blocks][page][R + dr], one row a token; for the matrix cores a second copy of
+// the latents, transposed a page at a time, [blocks][R][page]: the product with the values contracts over the keys, and
+// an MFMA operand wants consecutive entries of the contraction in one lane, so consecutive keys of one latent entry
+// must lie next to each other (the same reason the key/value cache keeps its values transposed).
 //
 //   latent_post    from the step's projections: RMS norm of the latent (float), rotation of the shared key part and
 //                  of every head's rotated query part (pairs (2i, 2i+1), float angles from a table), the latent row
 //                  written to its cache slot, the rotated query part written beside the absorbed part
 //   latent_attn_ref  one wave per (token, head), keys in ascending tiles of 64, float arithmetic, any sizes: the
 //                  kernel of the 32-bit path and the reference beside the MFMA kernel
-//   latent_attn_mfma bf16: a workgroup takes 16 (token, head) rows of one request (heads fastest) and walks the keys in
-//                  blocks of 32 through LDS; each of its waves takes every fourth block and keeps its own
-//                  (max, sum, output); they meet in LDS at the end. With `splits` > 1 the keys of a request are cut
-//                  into that many parts on the device (single rows: decode) and a merge kernel joins them.
+//   latent_attn_mfma bf16: a workgroup takes 16 (token, head) rows of one request (heads fastest); its four waves
+//                  deal the blocks of 32 keys among themselves in contiguous runs, each keeps its own (max, sum,
+//                  output), and they meet in LDS at the end. Scores are computed transposed (keys x rows), so that a
+//                  lane's eight weights are exactly its operand of the product with the values: nothing crosses lanes
+//                  between the two products, and a lane keeps the softmax state of one row. With `splits` > 1 the
+//                  keys of a request are cut into that many parts on the device (steps of single rows) and a merge
+//                  kernel joins them; the launch shape follows the step's counts alone.
 #include "common.cuh"
 
 using namespace dinfer;
@@ -34,7 +40,7 @@ __global__ void __launch_bounds__(256) latent_post_kernel(
     const S* __restrict__ proj, int64_t ld, int q_off, int c_off, int H, int dn, int dr, int R,
     const void* __restrict__ gain, int wf32, float eps, const int32_t* __restrict__ positions,
     const float* __restrict__ cos_sin, int rot, S* __restrict__ qa, int64_t ld_qa, S* __restrict__ cache,
-    const int64_t* __restrict__ slots) {
+    S* __restrict__ cache_t, int page, const int64_t* __restrict__ slots) {
   __shared__ float red[16];
   const int64_t t = blockIdx.x;
   const S* row = proj + t * ld;
@@ -69,7 +75,12 @@ __global__ void __launch_bounds__(256) latent_post_kernel(
   ss = block_sum(ss, red);
   const float inv = 1.f / sqrtf(ss / (float)R + eps);
   S* dst = cache + slot * (int64_t)(R + dr);
-  for (int i = threadIdx.x; i < R; i += blockDim.x) dst[i] = from_f32<S>(to_f32(c[i]) * inv * ld_param<S>(gain, i, wf32));
+  S* dst_t = cache_t ? cache_t + (slot / page) * (int64_t)R * page + (slot % page) : nullptr;
+  for (int i = threadIdx.x; i < R; i += blockDim.x) {
+    const S v = from_f32<S>(to_f32(c[i]) * inv * ld_param<S>(gain, i, wf32));
+    dst[i] = v;
+    if (dst_t) dst_t[(int64_t)i * page] = v;
+  }
   for (int j = threadIdx.x; j < pairs; j += blockDim.x) {
     float u = to_f32(c[R + 2 * j]), v = to_f32(c[R + 2 * j + 1]);
     if (cs && j < half) {
@@ -161,6 +172,220 @@ __global__ void __launch_bounds__(WAVES * 64) latent_attn_ref_kernel(
   }
 }
 
+
+// ---- attention over the latent pages on the matrix cores --------------------------------------------------------
+constexpr float LOG2E = 1.4426950408889634f;
+
+__device__ __forceinline__ f32x4 mfma16(bf16x8 a, bf16x8 b, f32x4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+}
+__device__ __forceinline__ float exp2_of(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// NT: tiles of 16 latent entries (R <= 16 NT, R a multiple of 16); the key rows are cut into NT / 2 + 4 chunks of 32
+// entries (dr <= 128). v_mfma_f32_16x16x32_bf16: lane l holds row (first operand) or column (second) l % 16 and the 8
+// entries of the contraction that belong to group l / 16; of the result, column l % 16 and rows 4 (l / 16) .. + 3.
+//   scores   first operand 16 keys x 32 key entries (rows of the cache, 16 bytes a lane), second the queries;
+//            lane l gets, for query row l % 16, the keys 4 (l / 16) .. + 3 of each of the block's two key tiles
+//   values   contraction over the block's 32 keys in the order (group g: keys 4g .. 4g+3 of the first tile, then of the
+//            second), which is the order in which a lane holds its weights; first operand 16 latent entries x those keys
+//            (two 8-byte pieces of the transposed pages), second the weights; the result is O^T: lane l holds query
+//            row l % 16 and latent entries 16 tile + 4 (l / 16) .. + 3.
+template <int NT>
+__global__ void __launch_bounds__(256) latent_attn_mfma_kernel(
+    const bf16* __restrict__ qa, int64_t ld_qa, bf16* __restrict__ out, int64_t ld_out, float* __restrict__ part,
+    const bf16* __restrict__ cache, const bf16* __restrict__ cache_t, const int32_t* __restrict__ block_table,
+    int64_t max_blocks, const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ seq_lens, int num_reqs,
+    float scale_log2, int window, int H, int R, int dr, int page, int splits) {
+  constexpr int NC = NT / 2 + 4;
+  extern __shared__ float meet[];   // [16][R + 2]: one wave's output, max and sum on their way to wave 0
+  // which request and which of its row tiles
+  int tile = blockIdx.x, b = 0, q_len = 0;
+  for (; b < num_reqs; ++b) {
+    q_len = cu_seqlens[b + 1] - cu_seqlens[b];
+    const int tiles = (q_len * H + 15) >> 4;
+    if (tile < tiles) break;
+    tile -= tiles;
+  }
+  if (b >= num_reqs) return;   // (the whole workgroup)
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, lr = lane & 15, g = lane >> 4;
+  const int DK = R + dr;
+  const int start = seq_lens[b] - q_len;
+  const int row0 = tile * 16;
+  const int nrows = q_len * H - row0 < 16 ? q_len * H - row0 : 16;
+  const bool rv = lr < nrows;
+  const int tok = rv ? (row0 + lr) / H : 0, head = rv ? (row0 + lr) % H : 0;
+  const int p = rv ? start + tok : -1;
+  const int p_first = start + row0 / H, p_last = start + (row0 + nrows - 1) / H;
+  const int first = window > 0 ? (p_first - window + 1 > 0 ? p_first - window + 1 : 0) : 0;
+  const int lowest = window > 0 ? (p - window + 1 > 0 ? p - window + 1 : 0) : 0;   // of this lane's row
+  const int kb0 = first & ~31;
+  const int nblk = (p_last - kb0) / 32 + 1;
+  const int parts = splits * 4, me = blockIdx.y * 4 + wave;
+  const int per = (nblk + parts - 1) / parts;
+  const int blk_lo = me * per, blk_hi = blk_lo + per < nblk ? blk_lo + per : nblk;
+  const int32_t* bt = block_table + (int64_t)b * max_blocks;
+
+  bf16x8 zero;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) zero[i] = (bf16)0.f;
+  bf16x8 qf[NC];
+  {
+    const bf16* qrow = qa + (int64_t)(cu_seqlens[b] + tok) * ld_qa + (int64_t)head * DK;
+#pragma unroll
+    for (int c = 0; c < NC; ++c) {
+      const int d = 32 * c + 8 * g;
+      qf[c] = (rv && d < DK) ? *(const bf16x8*)(qrow + d) : zero;
+    }
+  }
+  f32x4 o[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t) o[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, l = 0.f;
+
+  for (int blk = blk_lo; blk < blk_hi; ++blk) {
+    const int kb = kb0 + blk * 32;
+    f32x4 s[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      int key = kb + 16 * t + lr;
+      key = key < first ? first : (key > p_last ? p_last : key);   // a row that exists; what lies outside is masked below
+      const bf16* krow = cache + ((int64_t)bt[key / page] * page + (key % page)) * DK + 8 * g;
+      f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int c = 0; c < NC; ++c) {
+        if (32 * c < DK) {
+          const bf16x8 a = (32 * c + 8 * g < DK) ? *(const bf16x8*)(krow + 32 * c) : zero;
+          acc = mfma16(a, qf[c], acc);
+        }
+      }
+      s[t] = acc;
+    }
+    float mx = -INFINITY;
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int key = kb + 16 * t + 4 * g + i;
+        const float v = (key <= p && key >= lowest) ? s[t][i] * scale_log2 : -INFINITY;
+        s[t][i] = v;
+        mx = fmaxf(mx, v);
+      }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float m_new = fmaxf(m, mx);
+    const float alpha = m == -INFINITY ? 0.f : exp2_of(m - m_new);
+    bf16x8 pb;
+    float psum = 0.f;
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float pv = s[t][i] == -INFINITY ? 0.f : exp2_of(s[t][i] - m_new);
+        psum += pv;
+        pb[4 * t + i] = (bf16)pv;
+      }
+    l = l * alpha + psum;   // this lane's share of the row's sum; the four shares meet after the walk
+    m = m_new;
+    // the latents of keys kb + 4g .. + 3 and kb + 16 + 4g .. + 3, one latent entry a lane
+    const bf16* vt[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      int key = kb + 16 * t + 4 * g;
+      const int lo4 = first & ~3, hi4 = p_last & ~3;
+      key = key < lo4 ? lo4 : (key > hi4 ? hi4 : key);
+      vt[t] = cache_t + (int64_t)bt[key / page] * R * page + (key % page);
+    }
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      if (16 * t < R) {
+        const int64_t d = 16 * t + lr;
+        const bf16x4 a0 = *(const bf16x4*)(vt[0] + d * page);
+        const bf16x4 a1 = *(const bf16x4*)(vt[1] + d * page);
+        bf16x8 a;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) { a[i] = a0[i]; a[4 + i] = a1[i]; }
+        o[t] = mfma16(a, pb, o[t] * alpha);
+      }
+    }
+  }
+  l += __shfl_xor(l, 16, 64);
+  l += __shfl_xor(l, 32, 64);
+
+  // the waves meet: one after the other hands its state to wave 0
+  const int ldm = R + 2;
+  for (int w = 1; w < 4; ++w) {
+    if (wave == w) {
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+        if (16 * t < R)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) meet[lr * ldm + 16 * t + 4 * g + i] = o[t][i];
+      if (g == 0) { meet[lr * ldm + R] = m; meet[lr * ldm + R + 1] = l; }
+    }
+    __syncthreads();
+    if (wave == 0) {
+      const float m2 = meet[lr * ldm + R], l2 = meet[lr * ldm + R + 1];
+      const float mt = fmaxf(m, m2);
+      const float a1 = m == -INFINITY ? 0.f : exp2_of(m - mt), a2 = m2 == -INFINITY ? 0.f : exp2_of(m2 - mt);
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+        if (16 * t < R)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) o[t][i] = o[t][i] * a1 + meet[lr * ldm + 16 * t + 4 * g + i] * a2;
+      l = l * a1 + l2 * a2;
+      m = mt;
+    }
+    __syncthreads();
+  }
+  if (wave != 0 || !rv) return;
+  const int64_t trow = cu_seqlens[b] + tok;
+  if (splits == 1) {
+    const float inv = l > 0.f ? 1.f / l : 0.f;
+    bf16* orow = out + trow * ld_out + (int64_t)head * R;
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+      if (16 * t < R) {
+        bf16x4 y;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) y[i] = (bf16)(o[t][i] * inv);
+        *(bf16x4*)(orow + 16 * t + 4 * g) = y;
+      }
+  } else {
+    float* pr = part + ((trow * H + head) * splits + blockIdx.y) * (int64_t)ldm;
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+      if (16 * t < R)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) pr[16 * t + 4 * g + i] = o[t][i];
+    if (g == 0) { pr[R] = m; pr[R + 1] = l; }
+  }
+}
+
+// One workgroup per (token, head) row: the parts' (max, sum, output) become the row's output.
+__global__ void __launch_bounds__(128) latent_attn_merge_kernel(const float* __restrict__ part, bf16* __restrict__ out,
+                                                                int64_t ld_out, int H, int R, int splits) {
+  const int64_t row = blockIdx.x;
+  const int ldm = R + 2;
+  const float* pr = part + row * splits * (int64_t)ldm;
+  float mt = -INFINITY;
+  for (int s = 0; s < splits; ++s) mt = fmaxf(mt, pr[s * (int64_t)ldm + R]);
+  float lt = 0.f;
+  for (int s = 0; s < splits; ++s) {
+    const float ms = pr[s * (int64_t)ldm + R];
+    if (ms != -INFINITY) lt += pr[s * (int64_t)ldm + R + 1] * exp2_of(ms - mt);
+  }
+  const float inv = lt > 0.f ? 1.f / lt : 0.f;
+  bf16* orow = out + (row / H) * ld_out + (row % H) * (int64_t)R;
+  for (int d = threadIdx.x; d < R; d += blockDim.x) {
+    float acc = 0.f;
+    for (int s = 0; s < splits; ++s) {
+      const float ms = pr[s * (int64_t)ldm + R];
+      if (ms != -INFINITY) acc += pr[s * (int64_t)ldm + d] * exp2_of(ms - mt);
+    }
+    orow[d] = (bf16)(acc * inv);
+  }
+}
+
 }  // namespace
 
 // proj [T, ld]: the queries at column q_off (head h at h*(dn+dr): dn unrotated, then dr rotated), the down projection
@@ -170,15 +395,15 @@ __global__ void __launch_bounds__(WAVES * 64) latent_attn_ref_kernel(
 extern "C" int dinfer_latent_post(int dtype, const void* proj, int64_t tokens, int64_t ld, int q_off, int c_off, int heads,
                                   int dn, int dr, int R, const void* gain, int w_f32, float eps,
                                   const int32_t* positions, const float* cos_sin, int rot, void* qa, int64_t ld_qa,
-                                  void* cache, const int64_t* slots, hipStream_t stream) {
+                                  void* cache, void* cache_t, int page_size, const int64_t* slots, hipStream_t stream) {
   if (tokens <= 0) return OK;
   if (heads <= 0 || dn < 0 || dr < 0 || R <= 0 || rot < 0 || rot > dr || (rot & 1) || tokens > 0x7fffffff ||
-      ld_qa < (int64_t)heads * (R + dr))
+      ld_qa < (int64_t)heads * (R + dr) || (cache_t && page_size <= 0))
     return ERR_BAD_SHAPE;
   DINFER_DISPATCH_DTYPE(dtype, {
     latent_post_kernel<S><<<(unsigned)tokens, 256, 0, stream>>>((const S*)proj, ld, q_off, c_off, heads, dn, dr, R, gain,
                                                                w_f32, eps, positions, cos_sin, rot, (S*)qa, ld_qa,
-                                                               (S*)cache, slots);
+                                                               (S*)cache, (S*)cache_t, page_size, slots);
   });
   return launch_status();
 }
@@ -199,5 +424,45 @@ extern "C" int dinfer_latent_attn_ref(int dtype, const void* qa, int64_t ld_qa, 
                                                                  block_table, max_blocks, cu_seqlens, seq_lens,
                                                                  num_reqs, scale, window, heads, R, dr, page_size);
   });
+  return launch_status();
+}
+
+// Whether latent_attn_mfma takes these sizes.
+extern "C" int dinfer_latent_mfma_supports(int R, int dr, int page_size) {
+  return R >= 16 && R <= 512 && R % 16 == 0 && dr >= 0 && dr <= 128 && dr % 8 == 0 && page_size > 0 && page_size % 8 == 0;
+}
+
+// bf16. cache [blocks, page, R + dr] and cache_t [blocks, R, page]. splits > 1: every request brings one row; part holds
+// tokens * heads * splits * (R + 2) floats.
+extern "C" int dinfer_latent_attn_mfma(const void* qa, int64_t ld_qa, void* out, int64_t ld_out, float* part,
+                                       int64_t part_floats, const void* cache, const void* cache_t,
+                                       const int32_t* block_table, int64_t max_blocks, const int32_t* cu_seqlens,
+                                       const int32_t* seq_lens, int num_reqs, int64_t tokens, float scale, int window,
+                                       int heads, int R, int dr, int page_size, int splits, hipStream_t stream) {
+  if (tokens <= 0 || num_reqs <= 0) return OK;
+  if (heads <= 0 || max_blocks <= 0 || window < 0 || tokens > 0x7fffffff || splits < 1 || ld_qa % 8 || ld_out % 4 ||
+      ((uintptr_t)qa % 16) || ((uintptr_t)out % 8) || ((uintptr_t)cache % 16) || ((uintptr_t)cache_t % 8))
+    return ERR_BAD_SHAPE;
+  if (!dinfer_latent_mfma_supports(R, dr, page_size)) return ERR_UNSUPPORTED;
+  if (splits > 1 && (tokens != num_reqs || !part || part_floats < tokens * heads * splits * (int64_t)(R + 2)))
+    return ERR_WORKSPACE;
+  const int64_t tiles = (tokens * heads + 15) / 16 + num_reqs;
+  if (tiles > 0x7fffffff || splits > 65535) return ERR_UNSUPPORTED;
+  const dim3 grid((unsigned)tiles, (unsigned)splits);
+  const size_t lds = (size_t)16 * (R + 2) * sizeof(float);
+  const float sl = scale * LOG2E;
+#define LAUNCH(NT)                                                                                                     \
+  latent_attn_mfma_kernel<NT><<<grid, 256, lds, stream>>>((const bf16*)qa, ld_qa, (bf16*)out, ld_out, part,           \
+                                                          (const bf16*)cache, (const bf16*)cache_t, block_table,       \
+                                                          max_blocks, cu_seqlens, seq_lens, num_reqs, sl, window, heads, \
+                                                          R, dr, page_size, splits)
+  if (R <= 64) LAUNCH(4);
+  else if (R <= 128) LAUNCH(8);
+  else if (R <= 256) LAUNCH(16);
+  else LAUNCH(32);
+#undef LAUNCH
+  if (launch_status() != OK) return ERR_LAUNCH;
+  if (splits > 1)
+    latent_attn_merge_kernel<<<(unsigned)(tokens * heads), 128, 0, stream>>>(part, (bf16*)out, ld_out, heads, R, splits);
   return launch_status();
 }

@@ -1,7 +1,7 @@
 """Chooses the latent-attention kernels for a step.
 
 float32 storage: always the plain kernel (fixed key order, any sizes). bfloat16 storage: the MFMA kernel where the
-sizes fit it (latent and rotated part multiples of 32 and 8), with the keys of single rows cut into parts on the
+sizes fit it (latent a multiple of 16 up to 512, rotated part a multiple of 8 up to 128, pages of a multiple of 8), with the keys of single rows cut into parts on the
 device; the plain kernel otherwise.
 """
 from __future__ import annotations
@@ -20,13 +20,12 @@ class Workspace:
 
     def __init__(self, ctx, heads: int, rank: int, rot_dim: int):
         self.heads, self.rank, self.rot_dim = heads, rank, rot_dim
-        self.mfma = ctx.dtype == torch.bfloat16 and ops.latent_mfma_supports(rank, rot_dim)
+        self.mfma = ctx.dtype == torch.bfloat16 and ops.latent_mfma_supports(rank, rot_dim, ctx.page_size)
         longest = ctx.max_seq_len or 4096
         self.max_splits = max(1, min(MAX_SPLITS, -(-longest // SHORTEST_PART)))
         self.part = None
         if self.mfma:
-            tiles = -(-heads // 16)
-            units = max(self.splits(n) * n for n in range(1, ctx.max_reqs + 1)) * tiles * 16
+            units = max(self.splits(n) * n for n in range(1, ctx.max_reqs + 1)) * heads
             self.part = ctx.workspace.buffer("latent_partials", units * (rank + 2), dtype=torch.float32, rows=1)
 
     def splits(self, num_reqs: int) -> int:
@@ -35,7 +34,7 @@ class Workspace:
         return max(1, min(self.max_splits, TARGET_WORKGROUPS // max(1, num_reqs * tiles)))
 
 
-def paged_attention(qa: torch.Tensor, out: torch.Tensor, cache: torch.Tensor, batch, group: int, ws: Workspace, *,
+def paged_attention(qa: torch.Tensor, out: torch.Tensor, cache: torch.Tensor, cache_t, batch, group: int, ws: Workspace, *,
                     scale: float, window: int, heads: int, rank: int, rot_dim: int, page_size: int):
     """qa [T, heads * (rank + rot_dim)] -> out [T, heads * rank] (the attention's output in latent space)."""
     geo = dict(scale=scale, window=window, heads=heads, rank=rank, rot_dim=rot_dim, page_size=page_size)
@@ -44,5 +43,4 @@ def paged_attention(qa: torch.Tensor, out: torch.Tensor, cache: torch.Tensor, ba
     if not ws.mfma:
         return ops.latent_attn_ref(qa, out, cache, bt, batch.cu_seqlens, batch.seq_lens, B, T, **geo)
     splits = ws.splits(B) if batch.all_decode else 1
-    return ops.latent_attn_mfma(qa, out, cache, bt, batch.cu_seqlens, batch.seq_lens, B, T, batch.max_q_len, splits,
-                                ws.part, **geo)
+    return ops.latent_attn_mfma(qa, out, cache, cache_t, bt, batch.cu_seqlens, batch.seq_lens, B, T, splits, ws.part, **geo)

@@ -27,7 +27,9 @@ SIGNATURES = {
     "dinfer_embedding_to": ("elementwise", [_I, _I, _P, _P, _P, _L, _L, _L, _F, _P, _P, _P]),
     "dinfer_act": ("elementwise", [_I, _I, _P, _L, _P, _L, _L, _L, _P]),
     "dinfer_layernorm": ("norm", [_P, _I, _P, _I, _P, _P, _P, _I, _P, _I, _L, _L, _L, _L, _F, _P]),
-    "dinfer_latent_post": ("latent", [_I, _P, _L, _L, _I, _I, _I, _I, _I, _I, _P, _I, _F, _P, _P, _I, _P, _L, _P, _P, _P]),
+    "dinfer_latent_post": ("latent", [_I, _P, _L, _L, _I, _I, _I, _I, _I, _I, _P, _I, _F, _P, _P, _I, _P, _L, _P, _P, _I, _P, _P]),
+    "dinfer_latent_mfma_supports": ("latent", [_I, _I, _I]),
+    "dinfer_latent_attn_mfma": ("latent", [_P, _L, _P, _L, _P, _L, _P, _P, _P, _L, _P, _P, _I, _L, _F, _I, _I, _I, _I, _I, _I, _P]),
     "dinfer_latent_attn_ref": ("latent", [_I, _P, _L, _P, _L, _P, _P, _L, _P, _P, _I, _L, _F, _I, _I, _I, _I, _I, _P]),
     "dinfer_heads_nt": ("grouped", [_I, _P, _L, _L, _P, _L, _L, _P, _L, _L, _L, _L, _L, _L, _P, _L, _P]),
     "dinfer_experts_nt": ("grouped", [_I, _I, _P, _L, _P, _L, _L, _P, _L, _L, _L, _P, _L, _P, _P, _I, _I, _P]),

@@ -205,11 +205,12 @@ def latent_cache_shape(blocks: int, page_size: int, rank: int, rot_dim: int) -> 
 def latent_post(proj: torch.Tensor, tokens: int, *, heads: int, dim: int, rot_dim: int, rank: int, q_off: int,
                 c_off: int | None, gain: torch.Tensor | None, eps: float, positions: torch.Tensor,
                 cos_sin: torch.Tensor | None, rotary_dim: int, qa: torch.Tensor, cache: torch.Tensor | None,
-                slot_mapping: torch.Tensor | None) -> None:
+                slot_mapping: torch.Tensor | None, cache_t: torch.Tensor | None = None) -> None:
     """From the step's projections: every head's rotated query part goes, rotated, into qa (head h at h*(rank+rot_dim),
     behind the rank entries the caller fills), and, where the layer has a down projection of its own (c_off), the
-    token's latent (RMS-normed with `gain`) and rotated shared key part go to its cache slot."""
-    _need_gpu(proj, gain, positions, cos_sin, qa, cache, slot_mapping)
+    token's latent (RMS-normed with `gain`) and rotated shared key part go to its cache slot (the latent also into
+    cache_t [blocks, rank, page], the pages transposed, where that is given)."""
+    _need_gpu(proj, gain, positions, cos_sin, qa, cache, slot_mapping, cache_t)
     assert proj.shape[0] >= tokens and qa.shape[0] >= tokens and qa.dtype == proj.dtype
     assert q_off + heads * (dim + rot_dim) <= proj.shape[1] and qa.shape[1] >= heads * (rank + rot_dim)
     assert positions.dtype == torch.int32 and positions.numel() >= tokens
@@ -220,12 +221,15 @@ def latent_post(proj: torch.Tensor, tokens: int, *, heads: int, dim: int, rot_di
         assert c_off + rank + rot_dim <= proj.shape[1] and gain is not None and gain.numel() == rank
         assert slot_mapping.dtype == torch.int64 and slot_mapping.numel() >= tokens
         assert cache is not None and cache.dtype == proj.dtype and cache.is_contiguous()
-        assert cache.shape[-1] == rank + rot_dim
+        assert cache.shape[-1] == rank + rot_dim and cache.dim() == 3
+        if cache_t is not None:
+            assert cache_t.dtype == cache.dtype and cache_t.is_contiguous()
+            assert tuple(cache_t.shape) == (cache.shape[0], rank, cache.shape[1])
     lib.call("dinfer_latent_post", dtype_code(proj.dtype), proj.data_ptr(), tokens, _rows(proj), q_off,
              c_off if write else -1, heads, dim, rot_dim, rank, _ptr(gain) if write else 0,
              _is_param_f32(gain, proj.dtype) if write else 0, float(eps), positions.data_ptr(), _ptr(cos_sin),
              rotary_dim if cos_sin is not None else 0, qa.data_ptr(), _rows(qa), _ptr(cache) if write else 0,
-             _ptr(slot_mapping) if write else 0, _stream())
+             _ptr(cache_t) if write else 0, cache.shape[1] if write else 0, _ptr(slot_mapping) if write else 0, _stream())
 
 
 def _check_latent(qa, out, cache, block_table, cu_seqlens, seq_lens, num_reqs, tokens, heads, rank, rot_dim, page_size):
@@ -252,8 +256,28 @@ def latent_attn_ref(qa: torch.Tensor, out: torch.Tensor, cache: torch.Tensor, bl
     return out
 
 
-def latent_mfma_supports(rank: int, rot_dim: int) -> bool:
-    return False
+def latent_mfma_supports(rank: int, rot_dim: int, page_size: int) -> bool:
+    return bool(lib.get("dinfer_latent_mfma_supports")(rank, rot_dim, page_size))
+
+
+def latent_attn_mfma(qa: torch.Tensor, out: torch.Tensor, cache: torch.Tensor, cache_t: torch.Tensor,
+                     block_table: torch.Tensor, cu_seqlens: torch.Tensor, seq_lens: torch.Tensor, num_reqs: int,
+                     tokens: int, splits: int, part: torch.Tensor | None, *, scale: float, window: int, heads: int,
+                     rank: int, rot_dim: int, page_size: int) -> torch.Tensor:
+    """latent_attn_ref on the matrix cores (bfloat16): cache_t [blocks, rank, page] holds the latents once more, the
+    pages transposed. splits > 1 (steps in which every request brings one row): each request's keys are cut into that
+    many parts on the device and merged; part: float32 scratch of tokens * heads * splits * (rank + 2)."""
+    _need_gpu(qa, out, cache, cache_t, block_table, cu_seqlens, seq_lens, part)
+    _check_latent(qa, out, cache, block_table, cu_seqlens, seq_lens, num_reqs, tokens, heads, rank, rot_dim, page_size)
+    assert qa.dtype == torch.bfloat16 and cache_t.dtype == torch.bfloat16 and cache_t.is_contiguous()
+    assert tuple(cache_t.shape) == (cache.shape[0], rank, page_size)
+    if splits > 1:
+        assert part is not None and part.dtype == torch.float32 and part.is_contiguous() and tokens == num_reqs
+    lib.call("dinfer_latent_attn_mfma", qa.data_ptr(), _rows(qa), out.data_ptr(), _rows(out), _ptr(part),
+             part.numel() if part is not None else 0, cache.data_ptr(), cache_t.data_ptr(), block_table.data_ptr(),
+             block_table.shape[1], cu_seqlens.data_ptr(), seq_lens.data_ptr(), num_reqs, tokens, float(scale),
+             int(window), heads, rank, rot_dim, page_size, int(splits), _stream())
+    return out
 
 
 # ---- many small products in one launch ---------------------------------------------------------------

@@ -59,7 +59,8 @@ class LatentAttention(Mixer):
             raise ValueError("latent attention norms its latent by root mean square with a plain gain")
 
     def cache_spec(self):
-        return LatentSpec(self.rank, self.rot_dim, self.window)
+        # (asked after bind: the matrix-core kernel wants the latents a second time, transposed)
+        return LatentSpec(self.rank, self.rot_dim, self.window, transposed=self.attn_ws.mfma)
 
     def tensors(self):
         n, H = self.names, self.heads
@@ -113,9 +114,11 @@ class LatentAttention(Mixer):
         ops.latent_post(self.proj_buf, T, heads=H, dim=dn, rot_dim=dr, rank=R, q_off=0, c_off=self.c_off if write else None,
                         gain=gain, eps=self.latent_norm.eps if write else 0.0, positions=batch.positions,
                         cos_sin=self.position.table(), rotary_dim=self.position.rotary_dim, qa=self.qa_buf,
-                        cache=cache.latent if write else None, slot_mapping=batch.slot_mapping[g] if write else None)
+                        cache=cache.latent if write else None, slot_mapping=batch.slot_mapping[g] if write else None,
+                        cache_t=cache.tensors.get("latent_t") if write else None)
         ops.heads_nt(self.proj_buf, 0, dn + dr, self.uk_t, self.qa_buf, 0, R + dr, T)
-        latent_kernels.paged_attention(self.qa_buf, self.ol_buf, cache.latent, batch, g, self.attn_ws, scale=self.scale,
+        latent_kernels.paged_attention(self.qa_buf, self.ol_buf, cache.latent, cache.tensors.get("latent_t"), batch, g,
+                                       self.attn_ws, scale=self.scale,
                                        window=self.window or 0, heads=H, rank=R, rot_dim=dr, page_size=self.page_size)
         ops.heads_nt(self.ol_buf, 0, R, self.uv, self.attn_buf, 0, self.vdim, T,
                      gate=self.proj_buf if self.gated else None, gate_off=self.g_off)

@@ -105,22 +105,28 @@ class KVSpec(CacheSpec):
 @dataclass(frozen=True)
 class LatentSpec(CacheSpec):
     """Cache need of a mixer that stores one row a token which all its heads share: `rank` numbers of a latent from
-    which keys and values are made, and `rot_dim` numbers of a rotated key part. Pages [blocks, page, rank + rot_dim]."""
+    which keys and values are made, and `rot_dim` numbers of a rotated key part. Pages [blocks, page, rank + rot_dim];
+    transposed: the latents once more as [blocks, rank, page], which the matrix-core kernel's product with the values
+    reads (the contraction runs over the keys there)."""
     rank: int
     rot_dim: int
     window: int | None = None
+    transposed: bool = False
 
     def group_key(self) -> tuple:
-        return ("latent", self.rank, self.rot_dim, self.window)
+        return ("latent", self.rank, self.rot_dim, self.window, self.transposed)
 
     def page_bytes(self, page_size, dtype):
-        return (self.rank + self.rot_dim) * page_size * _element_size(dtype)
+        return ((2 if self.transposed else 1) * self.rank + self.rot_dim) * page_size * _element_size(dtype)
 
     def allocate(self, num_blocks, page_size, num_slots, dtype, device):
         import torch
         from ..kernels import ops
         shape = ops.latent_cache_shape(num_blocks, page_size, self.rank, self.rot_dim)
-        return {"latent": torch.zeros(shape, dtype=dtype, device=device)}
+        out = {"latent": torch.zeros(shape, dtype=dtype, device=device)}
+        if self.transposed:
+            out["latent_t"] = torch.zeros((num_blocks, self.rank, page_size), dtype=dtype, device=device)
+        return out
 
 
 @dataclass(frozen=True)

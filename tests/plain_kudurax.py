@@ -99,10 +99,19 @@ def gated_expert(h, w, p):
     return (a * torch.sigmoid(a) * (h @ w[p + "up"].to(F).T)) @ w[p + "down"].to(F).T
 
 
-def routed_ff(h, w, p, mlp):
+def routed_ff(h, w, p, mlp, forced=None):
+    """forced [T, k]: experts to use instead of the k best. Where rounding makes a close call go the other way the
+    rest of the computation can still be judged; every forced expert must be within a hair of the k best."""
     E, k = mlp["router"]["experts"], mlp["router"]["top"]
     z = h @ w[p + "router"].to(F).T
-    top, idx = z.topk(k, dim=-1)
+    idx = torch.argsort(-z, dim=-1, stable=True)[:, :k]      # the k largest; among equals the lowest index
+    if forced is not None:
+        kth = torch.gather(z, 1, idx)[:, -1:]
+        behind = (kth - torch.gather(z, 1, forced)).max().item()
+        assert behind <= 0.08 * z.std().item(), f"a forced expert is {behind:.3f} behind the k-th best: no close call"
+        assert all(len(set(row)) == k for row in forced.tolist()), "an expert is chosen twice"
+        idx = forced
+    top = torch.gather(z, 1, idx)
     share = torch.softmax(top, dim=-1)
     out = torch.zeros_like(h)
     for e in range(E):
@@ -114,9 +123,11 @@ def routed_ff(h, w, p, mlp):
     return out
 
 
-def forward(cfg: dict, w: dict, tokens, start: int = 0, latents: dict | None = None, layers_out: list | None = None):
+def forward(cfg: dict, w: dict, tokens, start: int = 0, latents: dict | None = None, layers_out: list | None = None,
+            choices: dict | None = None):
     """Logits [T, vocab] of one sequence's tokens at positions start.. . latents: layer -> (c, kr) of the positions
-    before `start`, extended in place, so that a sequence can be fed in pieces."""
+    before `start`, extended in place, so that a sequence can be fed in pieces. choices: layer -> [T, k] experts that
+    its routed feed-forward is to use (see routed_ff)."""
     eps = cfg["norm"]["eps"]
     tokens = torch.as_tensor(tokens, dtype=torch.long)
     T = tokens.numel()
@@ -139,7 +150,8 @@ def forward(cfg: dict, w: dict, tokens, start: int = 0, latents: dict | None = N
         mlp = layer.get("mlp")
         if mlp is not None:
             h = layer_norm(x, w[p + "norm2"].to(F), w[p + "norm2.b"].to(F), eps)
-            x = x + (dense_ff(h, w, p + "mlp.") if mlp["kind"] == "dense" else routed_ff(h, w, p + "mlp.", mlp))
+            forced = None if choices is None else choices.get(i)
+            x = x + (dense_ff(h, w, p + "mlp.") if mlp["kind"] == "dense" else routed_ff(h, w, p + "mlp.", mlp, forced))
         if layers_out is not None:
             layers_out.append(x.clone())
     x = layer_norm(x, w["final.norm"].to(F), w["final.norm.b"].to(F), eps)
