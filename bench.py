@@ -4,6 +4,7 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--layers L] [--shape 8b|14b|32b|0.6b]
                     [--prompt P] [--context C] [--workload decode|serving [--sampled]]
     python bench.py --workload closed --shape 0.6b --concurrency 8 --prompt 128 --max-tokens 128 [--num-requests N]
+    python bench.py --workload kudurax [--kudurax-shape 2k|4k] [--layers 4] [--prompt 2048] [--only kudurax|qwen3]
 
 Prints ONE JSON line. `value` is decoded tokens per second at the default batch (8), each
 request with a 2,048-token prompt in a 4,096-token context; a "step" is one decode step
@@ -197,6 +198,107 @@ def closed(a, torch, Engine, SamplingParams, Qwen3Config) -> int:
     return 0
 
 
+# Kudurax layer sizes that resemble a real model's (latent attention of 512 + 64 a token, 128 + 64 wide query heads,
+# a relu^2 feed-forward, routed experts with a shared one), and the Qwen3 layer of the same width beside each
+KUDURAX_SHAPES = {
+    "2k": dict(width=2048, heads=16, dim=128, rot_dim=64, vdim=128, rank=512, ff=8192, experts=64, top=6, expert_ff=1408,
+               shared_ff=2816, qwen=dict(num_attention_heads=16, num_key_value_heads=4, head_dim=128, intermediate_size=8192)),
+    "4k": dict(width=4096, heads=32, dim=128, rot_dim=64, vdim=128, rank=512, ff=12288, experts=64, top=8, expert_ff=1536,
+               shared_ff=3072, qwen=dict(num_attention_heads=32, num_key_value_heads=8, head_dim=128, intermediate_size=12288)),
+}
+
+
+def kudurax_config(shape: dict, layers: int, vocab: int) -> dict:
+    """Layers in fours: dense and routed feed-forwards in turn; the third and fourth read the second's cache."""
+    m = dict(heads=shape["heads"], dim=shape["dim"], rot_dim=shape["rot_dim"], vdim=shape["vdim"], kv_rank=shape["rank"],
+             scale=(shape["dim"] + shape["rot_dim"]) ** -0.5,
+             rot=dict(base=10000.0, dims=shape["rot_dim"], scaling=dict(factor=40.0, original=4096, fast=32.0, slow=1.0)))
+    dense = dict(kind="dense", ff=shape["ff"])
+    moe = dict(kind="moe", router=dict(experts=shape["experts"], top=shape["top"]), expert=dict(ff=shape["expert_ff"]),
+               shared=dict(ff=shape["shared_ff"]))
+    out = []
+    for i in range(layers):
+        mm = dict(m)
+        if i % 4 >= 2:
+            mm["kv_from"] = i - i % 4 + 1
+        out.append(dict(type="latent_attention", mixer=mm, mlp=moe if i % 2 else dense))
+    return dict(architecture="Kudurax", vocab=vocab, width=shape["width"], embedding=dict(scale=1.0), norm=dict(eps=1e-5),
+                layers=out)
+
+
+def kudurax(a, torch, Engine, SamplingParams) -> int:
+    """Prefill and decode throughput of Kudurax layers of a real model's sizes beside Qwen3 layers of the same width
+    (random weights, the same engine, the same steps): one JSON line with both."""
+    from dinfer_amd.config.kudurax import KuduraxConfig
+    from dinfer_amd.config.qwen3 import Qwen3Config
+    shape = KUDURAX_SHAPES[a.kudurax_shape]
+    layers, vocab, page = a.layers or 4, 32768, 16
+    PROMPT, CONTEXT = a.prompt, a.context
+    batches = [b for b in (1, 8, 64) if b * CONTEXT <= 64 * 4096]
+    models = {
+        "kudurax": KuduraxConfig.from_dict(kudurax_config(shape, layers, vocab)),
+        "qwen3": Qwen3Config.from_dict({**SIZES, "vocab_size": vocab, "hidden_size": shape["width"],
+                                        "num_hidden_layers": layers, **shape["qwen"]}),
+    }
+    rng = random.Random(0)
+    greedy = SamplingParams(max_tokens=CONTEXT - PROMPT, temperature=0.0, ignore_eos=True)
+    result = {}
+    for name, cfg in models.items():
+        if a.only and a.only != name:
+            continue
+        eng = Engine(config=cfg, seed=0, dtype=a.dtype, max_model_len=CONTEXT, max_num_seqs=max(batches),
+                     max_num_batched_tokens=PROMPT, block_size=page, num_blocks=max(batches) * CONTEXT // page + 64,
+                     hip_graph=not a.no_hip_graph)
+
+        def prompt():
+            return [rng.randrange(vocab) for _ in range(PROMPT)]
+
+        def time_prefill():
+            rid = eng.add_request(prompt(), greedy)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            eng.step()
+            torch.cuda.synchronize()
+            dt = time.perf_counter() - t0
+            eng.abort(rid)
+            return dt
+
+        time_prefill()
+        pre = min(time_prefill() for _ in range(3))
+        out = {"layers": layers, "prefill_tokens": PROMPT, "prefill_ms": round(pre * 1e3, 3),
+               "prefill_tok_s": round(PROMPT / pre, 1)}
+        for b in batches:
+            ids = [eng.add_request(prompt(), greedy) for _ in range(b)]
+            while any(r.num_computed < PROMPT for r in eng.scheduler.requests.values()):
+                eng.step()
+            for _ in range(a.warmup):
+                eng.step()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(a.steps):
+                eng.step()
+            torch.cuda.synchronize()
+            dt = (time.perf_counter() - t0) / a.steps
+            for i in ids:
+                eng.abort(i)
+            out[f"decode_b{b}_ms"] = round(dt * 1e3, 4)
+            out[f"decode_b{b}_tok_s"] = round(b / dt, 1)
+        result[name] = out
+        del eng
+        torch.cuda.empty_cache()
+    first = result.get("kudurax") or next(iter(result.values()))
+    print(json.dumps({
+        "metric": f"decode tok/s (Kudurax layers of width {shape['width']}, batch 8, {PROMPT}-token prompts)",
+        "value": first.get("decode_b8_tok_s"), "unit": "tokens/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": first.get("decode_b8_ms"), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16" if a.dtype == "bfloat16" else "fp32", "data": "synthetic",
+        "config": {"model": f"Kudurax layers ({a.kudurax_shape}), random weights, beside Qwen3 layers of the same width",
+                   "global_batch": 8, "seq_len": CONTEXT, "prompt_len": PROMPT, "parallelism": "single GPU",
+                   "layers": layers, "vocab": vocab, "page_size": page, "hip_graph": not a.no_hip_graph, **shape},
+        "models": result}))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -211,11 +313,14 @@ def main() -> int:
     ap.add_argument("--shape", default="8b", choices=sorted(SHAPES), help="layer sizes (default: Qwen3-8B)")
     ap.add_argument("--prompt", type=int, default=DEFAULT_PROMPT, help="prompt tokens per request (and of the timed prefill)")
     ap.add_argument("--context", type=int, default=DEFAULT_CONTEXT, help="max_model_len the engine is built for")
-    ap.add_argument("--workload", default="decode", choices=["decode", "serving", "closed"],
+    ap.add_argument("--kudurax-shape", default="2k", choices=sorted(KUDURAX_SHAPES), help="kudurax: layer sizes")
+    ap.add_argument("--only", default="", choices=["", "kudurax", "qwen3"], help="kudurax: measure one of the two models")
+    ap.add_argument("--workload", default="decode", choices=["decode", "serving", "closed", "kudurax"],
                     help="serving: 32 requests with prompts of 512 to 3,072 tokens fed in portions of 512 beside the "
                          "requests that decode, 256 outputs each (meant for the 14B shape); closed: --concurrency "
                          "requests live at any time, --prompt tokens in and --max-tokens out each, the load of the "
-                         "reference's own serving bench without the server; each its own JSON line")
+                         "reference's own serving bench without the server; kudurax: prefill and decode of Kudurax "
+                         "layers of a real model's sizes beside Qwen3 layers of the same width; each its own JSON line")
     ap.add_argument("--concurrency", type=int, default=8, help="closed: live requests")
     ap.add_argument("--max-tokens", type=int, default=128, help="closed: outputs per request")
     ap.add_argument("--num-requests", type=int, default=0, help="closed: requests in all (0: four per live request, at least 16)")
@@ -231,6 +336,8 @@ def main() -> int:
     import torch
     from dinfer_amd import Engine, SamplingParams
     from dinfer_amd.config.qwen3 import Qwen3Config
+    if a.workload == "kudurax":
+        return kudurax(a, torch, Engine, SamplingParams)
     if a.workload == "serving":
         return serving(a, torch, Engine, SamplingParams, Qwen3Config)
     if a.workload == "closed":

@@ -13,11 +13,12 @@
 //
 // Float operands run on the vector ALUs, every output element summed over k in ascending order by one thread (the
 // true 32-bit path; a row's result does not depend on which tile or group size it met). bf16 operands run on the
-// matrix cores: a workgroup of four waves takes 64 x 64 outputs, each wave a 16-row strip, operands read straight
-// from memory in the MFMA's own order (8 consecutive k a lane), float accumulation over ascending k.
+// matrix cores, operands read straight from memory in the MFMA's own order (8 consecutive k a lane), in two forms:
+// tiles of 128 rows (a wave 64 x 64 outputs) and tiles of 16 rows whose waves split k (see the kernels).
 //
-//   moe_route    router logits in float, the `top` largest (lowest index first among equals), softmax over the chosen,
-//                and the shared expert's sigmoid gate
+//   moe_route    two kernels: router logits in float (a wave an expert, a router row read once per 8 tokens), then per
+//                token the `top` largest (lowest index first among equals), the softmax over the chosen and the shared
+//                expert's sigmoid gate
 //   moe_scatter  counts, offsets, the sorted list and the work list, one workgroup (LDS counters)
 //   moe_combine  out[t] = sum_c share[t, c] * y[t * top + c] + shared_gate[t] * shared[t]
 #include "common.cuh"
@@ -38,6 +39,7 @@ struct Groups {
   int c_to_perm;            // experts: C row = perm[i] instead of i
   const void* gate; int64_t ld_gate;   // heads: optional
   int gate_n;               // GATED: rows of each half of W_g
+  int tm;                   // rows of a tile: 64 on the vector ALUs, 16 or 128 on the matrix cores
 };
 
 __device__ __forceinline__ float silu(float x) { return x / (1.f + expf(-x)); }
@@ -50,18 +52,19 @@ struct Tile {
   int z, m0, rows;
   const int32_t* perm; int a_div, c_to_perm, base;
   __device__ __forceinline__ bool init(const Groups& p) {
+    const int tm = p.tm;   // rows a tile
     if (p.tiles) {
       z = p.tiles[2 * blockIdx.y];
       if (z < 0) return false;
       base = p.tiles[2 * blockIdx.y + 1];
       m0 = 0;
       const int end = p.offsets[z + 1];
-      rows = end - base < BM ? end - base : BM;
+      rows = end - base < tm ? end - base : tm;
       perm = p.perm; a_div = p.a_div; c_to_perm = p.c_to_perm;
     } else {
       z = blockIdx.z;
-      m0 = blockIdx.y * BM;
-      rows = p.M - m0 < BM ? p.M - m0 : BM;
+      m0 = blockIdx.y * tm;
+      rows = p.M - m0 < tm ? p.M - m0 : tm;
       perm = nullptr; a_div = 0; c_to_perm = 0; base = m0;
     }
     return rows > 0;
@@ -144,106 +147,201 @@ __global__ void __launch_bounds__(256) grouped_valu_kernel(Groups p) {
   }
 }
 
-// bf16 on the matrix cores. A wave owns rows [16 w, 16 w + 16) of the tile and all 64 columns (four 16 x 16 outputs,
-// twice that when gated). v_mfma_f32_16x16x32_bf16: lane l holds row (or column) l % 16 and the 8 consecutive k
-// starting at 8 (l / 16); of the result it holds column l % 16, rows 4 (l / 16) .. + 3.
+// bf16 on the matrix cores. v_mfma_f32_16x16x32_bf16: lane l holds row (or column) l % 16 and the 8 consecutive k
+// starting at 8 (l / 16); of the result it holds column l % 16, rows 4 (l / 16) .. + 3. Operands are read straight from
+// memory in that order (16 bytes a lane).
+//
+// Many rows (tiles of 128): a workgroup takes 128 rows x 128 columns (gated: 64 columns of each half), its waves
+// 2 x 2, a wave 64 x 64: four row fragments and four column fragments feed sixteen MFMAs a step of 32 k.
+constexpr int TM_BIG = 128, TM_SMALL = 16;
+
 template <class O, bool GATED>
-__global__ void __launch_bounds__(256) grouped_mfma_kernel(Groups p) {
-  __shared__ int64_t arow[BM];
+__global__ void __launch_bounds__(256) grouped_mfma_big_kernel(Groups p) {
+  __shared__ int64_t arow[TM_BIG];
   Tile tl;
   if (!tl.init(p)) return;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int n0 = blockIdx.x * BN;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int n0 = blockIdx.x * (GATED ? 64 : 128);
   const bool experts = p.tiles != nullptr;
   const bf16* A = (const bf16*)p.A + (experts ? 0 : (int64_t)tl.z * p.a_zs);
   const bf16* W = (const bf16*)p.W + (int64_t)tl.z * p.w_zs;
-  if (threadIdx.x < BM) arow[threadIdx.x] = threadIdx.x < tl.rows ? tl.a_row(threadIdx.x) : -1;
+  if (threadIdx.x < TM_BIG) arow[threadIdx.x] = threadIdx.x < tl.rows ? tl.a_row(threadIdx.x) : -1;
   __syncthreads();
-  if (wave * 16 >= tl.rows) return;   // (no barrier follows)
+  if (wm * 64 >= tl.rows) return;   // (no barrier follows)
   const int lr = lane & 15, kq = lane >> 4;
-  const int64_t ar = arow[wave * 16 + lr];
-  const bf16* ap = ar >= 0 ? A + ar * p.lda + kq * 8 : nullptr;
+  const bf16* ap[4];
   const bf16* wp[4];
-  const bf16* up[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int64_t ar = arow[wm * 64 + i * 16 + lr];
+    ap[i] = ar >= 0 ? A + ar * p.lda + kq * 8 : nullptr;
+  }
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
-    const int gn = n0 + j * 16 + lr;
-    wp[j] = gn < p.N ? W + (int64_t)gn * p.ldw + kq * 8 : nullptr;
-    up[j] = (GATED && gn < p.N) ? W + (int64_t)(gn + p.gate_n) * p.ldw + kq * 8 : nullptr;
+    // gated: fragments 0, 1 are gate columns, 2, 3 the up columns of the same numbers
+    const int gn = GATED ? n0 + wn * 32 + (j & 1) * 16 + lr : n0 + wn * 64 + j * 16 + lr;
+    const int64_t wrow = GATED && j >= 2 ? gn + p.gate_n : gn;
+    wp[j] = gn < p.N ? W + wrow * p.ldw + kq * 8 : nullptr;
   }
   bf16x8 zero;
 #pragma unroll
   for (int i = 0; i < 8; ++i) zero[i] = (bf16)0.f;
-  f32x4 acc[4], acu[4];
+  f32x4 acc[4][4];
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
-    acu[j] = f32x4{0.f, 0.f, 0.f, 0.f};
-  }
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
   const int K = p.K;   // a multiple of 8 (checked on the host)
   for (int k0 = 0; k0 < K; k0 += 32) {
     const bool in = k0 + kq * 8 < K;
-    const bf16x8 a = (ap && in) ? *(const bf16x8*)(ap + k0) : zero;
+    bf16x8 a[4], w[4];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const bf16x8 w = (wp[j] && in) ? *(const bf16x8*)(wp[j] + k0) : zero;
-      acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, w, acc[j], 0, 0, 0);
-      if (GATED) {
-        const bf16x8 u = (up[j] && in) ? *(const bf16x8*)(up[j] + k0) : zero;
-        acu[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, u, acu[j], 0, 0, 0);
-      }
-    }
+    for (int i = 0; i < 4; ++i) a[i] = (ap[i] && in) ? *(const bf16x8*)(ap[i] + k0) : zero;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) w[j] = (wp[j] && in) ? *(const bf16x8*)(wp[j] + k0) : zero;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i], w[j], acc[i][j], 0, 0, 0);
   }
   O* C = (O*)p.C + (experts ? 0 : (int64_t)tl.z * p.c_zs);
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int r = wave * 16 + kq * 4 + i;
-    if (r >= tl.rows) continue;
-    const int64_t cr = tl.c_row(r);
-    float g = 1.f;
-    if (p.gate) g = sigmoid((float)((const bf16*)p.gate)[cr * p.ld_gate + tl.z]);
+  for (int i = 0; i < 4; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int gn = n0 + j * 16 + lr;
-      if (gn < p.N) {
-        const float v = GATED ? silu(acc[j][i]) * acu[j][i] : acc[j][i];
-        C[cr * p.ldc + gn] = from_f32<O>(v * g);
+    for (int r = 0; r < 4; ++r) {
+      const int row = wm * 64 + i * 16 + kq * 4 + r;
+      if (row >= tl.rows) continue;
+      const int64_t cr = tl.c_row(row);
+      float g = 1.f;
+      if (p.gate) g = sigmoid((float)((const bf16*)p.gate)[cr * p.ld_gate + tl.z]);
+#pragma unroll
+      for (int j = 0; j < (GATED ? 2 : 4); ++j) {
+        const int gn = GATED ? n0 + wn * 32 + j * 16 + lr : n0 + wn * 64 + j * 16 + lr;
+        if (gn < p.N) {
+          const float v = GATED ? silu(acc[i][j][r]) * acc[i][j + 2][r] : acc[i][j][r];
+          C[cr * p.ldc + gn] = from_f32<O>(v * g);
+        }
       }
     }
+}
+
+// Few rows (tiles of 16: steps of single tokens): time is the time to stream the weights, so a workgroup takes only 16
+// columns (gated: of each half) and its four waves take a quarter of k each; their partial sums meet in LDS and are
+// added in wave order.
+template <class O, bool GATED>
+__global__ void __launch_bounds__(256) grouped_mfma_small_kernel(Groups p) {
+  __shared__ int64_t arow[TM_SMALL];
+  __shared__ float part[4][GATED ? 2 : 1][16][17];
+  Tile tl;
+  if (!tl.init(p)) return;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int n0 = blockIdx.x * 16;
+  const bool experts = p.tiles != nullptr;
+  const bf16* A = (const bf16*)p.A + (experts ? 0 : (int64_t)tl.z * p.a_zs);
+  const bf16* W = (const bf16*)p.W + (int64_t)tl.z * p.w_zs;
+  if (threadIdx.x < TM_SMALL) arow[threadIdx.x] = threadIdx.x < tl.rows ? tl.a_row(threadIdx.x) : -1;
+  __syncthreads();
+  const int lr = lane & 15, kq = lane >> 4;
+  const int64_t ar = arow[lr];
+  const int gn = n0 + lr;
+  const bf16* ap = ar >= 0 ? A + ar * p.lda + kq * 8 : nullptr;
+  const bf16* wp = gn < p.N ? W + (int64_t)gn * p.ldw + kq * 8 : nullptr;
+  const bf16* up = (GATED && gn < p.N) ? W + (int64_t)(gn + p.gate_n) * p.ldw + kq * 8 : nullptr;
+  bf16x8 zero;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) zero[i] = (bf16)0.f;
+  const int K = p.K;
+  const int steps = (K + 31) / 32, per = (steps + 3) / 4;
+  const int k_lo = wave * per * 32, k_hi = (wave + 1) * per * 32 < K ? (wave + 1) * per * 32 : K;
+  f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f}, acu = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll 4
+  for (int k0 = k_lo; k0 < k_hi; k0 += 32) {
+    const bool in = k0 + kq * 8 < K;
+    const bf16x8 a = (ap && in) ? *(const bf16x8*)(ap + k0) : zero;
+    const bf16x8 w = (wp && in) ? __builtin_nontemporal_load((const bf16x8*)(wp + k0)) : zero;
+    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, w, acc, 0, 0, 0);
+    if (GATED) {
+      const bf16x8 u = (up && in) ? __builtin_nontemporal_load((const bf16x8*)(up + k0)) : zero;
+      acu = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, u, acu, 0, 0, 0);
+    }
   }
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    part[wave][0][kq * 4 + r][lr] = acc[r];
+    if (GATED) part[wave][GATED ? 1 : 0][kq * 4 + r][lr] = acu[r];
+  }
+  __syncthreads();
+  const int row = threadIdx.x >> 4, col = threadIdx.x & 15;
+  if (row >= tl.rows || n0 + col >= p.N) return;
+  float v = 0.f, u = 0.f;
+#pragma unroll
+  for (int w = 0; w < 4; ++w) {
+    v += part[w][0][row][col];
+    if (GATED) u += part[w][GATED ? 1 : 0][row][col];
+  }
+  const int64_t cr = tl.c_row(row);
+  float g = 1.f;
+  if (p.gate) g = sigmoid((float)((const bf16*)p.gate)[cr * p.ld_gate + tl.z]);
+  O* C = (O*)p.C + (experts ? 0 : (int64_t)tl.z * p.c_zs);
+  C[cr * p.ldc + n0 + col] = from_f32<O>((GATED ? silu(v) * u : v) * g);
 }
 
 // ---- routing ---------------------------------------------------------------------------------------------------
 constexpr int MAX_EXPERTS = 1024;
 
+// Router logits: a wave takes one expert (the row after the last expert is the shared expert's gate vector) and up to
+// RT tokens, so a router row is read once per RT tokens; a lane sums every 64th entry, then the lanes meet. z [T, ldz].
+constexpr int RT = 8;
+
 template <class S>
-__global__ void __launch_bounds__(256) moe_route_kernel(const S* __restrict__ x, int64_t ld_x, const float* __restrict__ wr,
-                                                        const float* __restrict__ wsg, int E, int top, int width,
-                                                        int32_t* __restrict__ idx, float* __restrict__ share,
-                                                        float* __restrict__ shared_gate) {
-  __shared__ float z[MAX_EXPERTS];
-  const int64_t t = blockIdx.x;
-  const S* xr = x + t * ld_x;
+__global__ void __launch_bounds__(256) moe_logits_kernel(const S* __restrict__ x, int64_t ld_x, int tokens,
+                                                         const float* __restrict__ wr, const float* __restrict__ wsg,
+                                                         int E, int width, float* __restrict__ z, int ldz) {
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  for (int e = wave; e < E + (wsg ? 1 : 0); e += 4) {
-    const float* w = e < E ? wr + (int64_t)e * width : wsg;
-    float acc = 0.f;
-    for (int i = lane; i < width; i += 64) acc = fmaf(to_f32(xr[i]), w[i], acc);
-    acc = wave_sum(acc);
-    if (lane == 0) {
-      if (e < E) z[e] = acc; else shared_gate[t] = sigmoid(acc);
-    }
+  const int e = blockIdx.y * 4 + wave;
+  if (e >= E + (wsg ? 1 : 0)) return;
+  const float* w = e < E ? wr + (int64_t)e * width : wsg;
+  const int t0 = blockIdx.x * RT;
+  const int nt = tokens - t0 < RT ? tokens - t0 : RT;
+  float acc[RT];
+#pragma unroll
+  for (int r = 0; r < RT; ++r) acc[r] = 0.f;
+#pragma unroll 4
+  for (int i = lane; i < width; i += 64) {
+    const float wv = w[i];
+#pragma unroll
+    for (int r = 0; r < RT; ++r)
+      if (r < nt) acc[r] = fmaf(to_f32(x[(int64_t)(t0 + r) * ld_x + i]), wv, acc[r]);
   }
-  __syncthreads();
-  if (wave != 0) return;
-  // the `top` largest, one after the other; among equals the lowest index
+#pragma unroll
+  for (int r = 0; r < RT; ++r) {
+    const float v = wave_sum(acc[r]);
+    if (lane == 0 && r < nt) z[(int64_t)(t0 + r) * ldz + e] = v;
+  }
+}
+
+// A wave per token: the `top` largest of its logits, one after the other (among equals the lowest index), the softmax
+// over the chosen, and the sigmoid of the shared expert's gate logit (z[t, E]) where there is one.
+__global__ void __launch_bounds__(256) moe_topk_kernel(const float* __restrict__ z, int ldz, int tokens, int E, int top,
+                                                       int has_shared, int32_t* __restrict__ idx,
+                                                       float* __restrict__ share, float* __restrict__ shared_gate) {
+  __shared__ float zs[4][MAX_EXPERTS];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int64_t t = (int64_t)blockIdx.x * 4 + wave;
+  if (t >= tokens) return;   // (no workgroup barrier below)
+  float* zw = zs[wave];
+  for (int e = lane; e < E; e += 64) zw[e] = z[t * ldz + e];
+  if (has_shared && lane == 0) shared_gate[t] = sigmoid(z[t * ldz + E]);
+  __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+  __builtin_amdgcn_wave_barrier();
   float chosen = 0.f, zmax = 0.f, sum = 0.f;   // lane c keeps the c-th choice
   int chosen_e = 0;
   for (int c = 0; c < top; ++c) {
     float best = -INFINITY;
     int be = 0x7fffffff;
     for (int e = lane; e < E; e += 64) {
-      const float v = z[e];
+      const float v = zw[e];
       if (v > best || (v == best && e < be)) { best = v; be = e; }
     }
 #pragma unroll
@@ -253,8 +351,8 @@ __global__ void __launch_bounds__(256) moe_route_kernel(const S* __restrict__ x,
       if (ov > best || (ov == best && oe < be)) { best = ov; be = oe; }
     }
     if (c == 0) zmax = best;
-    if (lane == (c & 63)) { chosen = best; chosen_e = be; }
-    if (lane == 0 && be < E) z[be] = -INFINITY;
+    if (lane == c) { chosen = best; chosen_e = be; }
+    if (lane == 0 && be < E) zw[be] = -INFINITY;
     __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
     __builtin_amdgcn_wave_barrier();
     sum += expf(best - zmax);   // every lane holds the same sum, added in the order of the choices
@@ -316,22 +414,57 @@ __global__ void __launch_bounds__(256) moe_combine_kernel(const S* __restrict__ 
   }
 }
 
-template <bool GATED>
-int launch_groups(int dtype, int out_f32, const Groups& p, dim3 grid, hipStream_t stream) {
-  if (dtype == DT_F32) {
-    grouped_valu_kernel<float, float, GATED><<<grid, 256, 0, stream>>>(p);
-  } else if (dtype == DT_BF16) {
-    const bool mfma = p.K % 8 == 0 && p.lda % 8 == 0 && p.ldw % 8 == 0 && p.a_zs % 8 == 0 && p.w_zs % 8 == 0 &&
-                      ((uintptr_t)p.A % 16) == 0 && ((uintptr_t)p.W % 16) == 0;
-    if (mfma) {
-      if (out_f32) grouped_mfma_kernel<float, GATED><<<grid, 256, 0, stream>>>(p);
-      else grouped_mfma_kernel<bf16, GATED><<<grid, 256, 0, stream>>>(p);
-    } else {
-      if (out_f32) grouped_valu_kernel<bf16, float, GATED><<<grid, 256, 0, stream>>>(p);
-      else grouped_valu_kernel<bf16, bf16, GATED><<<grid, 256, 0, stream>>>(p);
+inline bool mfma_fits(int dtype, const Groups& p) {
+  return dtype == DT_BF16 && p.K % 8 == 0 && p.lda % 8 == 0 && p.ldw % 8 == 0 && p.a_zs % 8 == 0 && p.w_zs % 8 == 0 &&
+         ((uintptr_t)p.A % 16) == 0 && ((uintptr_t)p.W % 16) == 0;
+}
+
+// grid.x is set here from the kernel's columns a workgroup; grid.y / z arrive from the caller (tiles, groups).
+// bf16 rows whose width is a multiple of 8: a thread takes 8 consecutive entries of every chosen expert's row.
+__global__ void __launch_bounds__(256) moe_combine_bf16x8_kernel(const bf16* __restrict__ y, int64_t ld_y,
+                                                                 const float* __restrict__ share, int top,
+                                                                 const bf16* __restrict__ shared, int64_t ld_s,
+                                                                 const float* __restrict__ shared_gate,
+                                                                 bf16* __restrict__ out, int64_t ld_o, int width) {
+  const int64_t t = blockIdx.x;
+  const float sg = shared ? shared_gate[t] : 0.f;
+  for (int i = threadIdx.x * 8; i < width; i += blockDim.x * 8) {
+    float acc[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[j] = 0.f;
+    for (int c = 0; c < top; ++c) {
+      const bf16x8 v = *(const bf16x8*)(y + (t * top + c) * ld_y + i);
+      const float w = share[t * top + c];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) acc[j] = fmaf(w, (float)v[j], acc[j]);
     }
+    if (shared) {
+      const bf16x8 v = *(const bf16x8*)(shared + t * ld_s + i);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) acc[j] = fmaf(sg, (float)v[j], acc[j]);
+    }
+    bf16x8 r;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) r[j] = (bf16)acc[j];
+    *(bf16x8*)(out + t * ld_o + i) = r;
+  }
+}
+
+template <bool GATED>
+int launch_groups(int dtype, Groups p, unsigned gy, unsigned gz, hipStream_t stream) {
+  if (dtype != DT_F32 && dtype != DT_BF16) return ERR_BAD_DTYPE;
+  if (mfma_fits(dtype, p) && p.tm == TM_SMALL) {
+    const dim3 grid((unsigned)((p.N + 15) / 16), gy, gz);
+    grouped_mfma_small_kernel<bf16, GATED><<<grid, 256, 0, stream>>>(p);
+  } else if (mfma_fits(dtype, p) && p.tm == TM_BIG) {
+    const int cols = GATED ? 64 : 128;
+    const dim3 grid((unsigned)((p.N + cols - 1) / cols), gy, gz);
+    grouped_mfma_big_kernel<bf16, GATED><<<grid, 256, 0, stream>>>(p);
   } else {
-    return ERR_BAD_DTYPE;
+    if (p.tm > BM) return ERR_UNSUPPORTED;
+    const dim3 grid((unsigned)((p.N + BN - 1) / BN), gy, gz);
+    if (dtype == DT_F32) grouped_valu_kernel<float, float, GATED><<<grid, 256, 0, stream>>>(p);
+    else grouped_valu_kernel<bf16, bf16, GATED><<<grid, 256, 0, stream>>>(p);
   }
   return launch_status();
 }
@@ -344,54 +477,69 @@ extern "C" int dinfer_heads_nt(int dtype, const void* A, int64_t lda, int64_t a_
                                int64_t groups, const void* gate, int64_t ld_gate, hipStream_t stream) {
   if (M <= 0 || N <= 0 || groups <= 0) return OK;
   if (K <= 0 || ldw < K || M > 0x7fffffff || N > 0x7fffffff || K > 0x7fffffff || groups > 65535) return ERR_BAD_SHAPE;
-  const int64_t gy = (M + BM - 1) / BM;
-  if (gy > 65535) return ERR_UNSUPPORTED;
   Groups p{};
   p.A = A; p.lda = lda; p.a_zs = a_zs; p.W = W; p.ldw = ldw; p.w_zs = w_zs; p.C = C; p.ldc = ldc; p.c_zs = c_zs;
   p.M = (int)M; p.N = (int)N; p.K = (int)K; p.gate = gate; p.ld_gate = ld_gate;
-  const dim3 grid((unsigned)((N + BN - 1) / BN), (unsigned)gy, (unsigned)groups);
-  return launch_groups<false>(dtype, 0, p, grid, stream);
+  p.tm = !mfma_fits(dtype, p) ? BM : M <= TM_SMALL ? TM_SMALL : TM_BIG;
+  const int64_t gy = (M + p.tm - 1) / p.tm;
+  if (gy > 65535) return ERR_UNSUPPORTED;
+  return launch_groups<false>(dtype, p, (unsigned)gy, (unsigned)groups, stream);
 }
 
 // The products of the experts (see the head of the file). W [experts][rows][ldw] with w_zs elements an expert;
 // gated != 0: rows = 2 N (gate rows, then up rows). max_tiles: the length of `tiles`.
 extern "C" int dinfer_experts_nt(int dtype, int gated, const void* A, int64_t lda, const void* W, int64_t ldw,
                                  int64_t w_zs, void* C, int64_t ldc, int64_t N, int64_t K, const int32_t* tiles,
-                                 int64_t max_tiles, const int32_t* offsets, const int32_t* perm, int a_div,
+                                 int64_t max_tiles, int tile_rows, const int32_t* offsets, const int32_t* perm, int a_div,
                                  int c_to_perm, hipStream_t stream) {
   if (N <= 0 || max_tiles <= 0) return OK;
   if (K <= 0 || ldw < K || lda < K || ldc < N || N > 0x7fffffff || K > 0x7fffffff || max_tiles > 65535 || !tiles ||
-      !offsets || !perm)
+      !offsets || !perm || tile_rows <= 0)
     return ERR_BAD_SHAPE;
   Groups p{};
   p.A = A; p.lda = lda; p.W = W; p.ldw = ldw; p.w_zs = w_zs; p.C = C; p.ldc = ldc;
   p.N = (int)N; p.K = (int)K; p.tiles = tiles; p.offsets = offsets; p.perm = perm; p.a_div = a_div;
-  p.c_to_perm = c_to_perm; p.gate_n = (int)N;
-  const dim3 grid((unsigned)((N + BN - 1) / BN), (unsigned)max_tiles, 1);
-  return gated ? launch_groups<true>(dtype, 0, p, grid, stream) : launch_groups<false>(dtype, 0, p, grid, stream);
+  p.c_to_perm = c_to_perm; p.gate_n = (int)N; p.tm = tile_rows;
+  if (!mfma_fits(dtype, p) && tile_rows > BM) return ERR_UNSUPPORTED;
+  return gated ? launch_groups<true>(dtype, p, (unsigned)max_tiles, 1, stream)
+               : launch_groups<false>(dtype, p, (unsigned)max_tiles, 1, stream);
 }
 
-extern "C" int dinfer_moe_tile_rows() { return BM; }
+// Rows of a tile for a routed layer's two products: the matrix-core kernels take 16 (few rows an expert: the weights
+// are streamed) or 128; anything else (float, sizes that are no multiples of 8) runs on the vector ALUs with 64.
+extern "C" int dinfer_moe_tile_rows(int dtype, int64_t entries, int experts, int64_t k_in, int64_t k_mid) {
+  if (dtype != DT_BF16 || k_in % 8 || k_mid % 8) return BM;
+  return entries <= (int64_t)TM_SMALL * experts ? TM_SMALL : TM_BIG;
+}
 
+
+// z: float scratch [tokens, experts + 1].
 extern "C" int dinfer_moe_route(int dtype, const void* x, int64_t ld_x, int64_t tokens, const float* router,
-                                const float* shared_gate_w, int experts, int top, int width, int32_t* idx, float* share,
-                                float* shared_gate, hipStream_t stream) {
+                                const float* shared_gate_w, int experts, int top, int width, float* z, int32_t* idx,
+                                float* share, float* shared_gate, hipStream_t stream) {
   if (tokens <= 0) return OK;
-  if (experts <= 0 || top <= 0 || top > experts || width <= 0 || tokens > 0x7fffffff) return ERR_BAD_SHAPE;
+  if (experts <= 0 || top <= 0 || top > experts || width <= 0 || tokens > 0x7fffffff || !z) return ERR_BAD_SHAPE;
   if (experts > MAX_EXPERTS || top > 64) return ERR_UNSUPPORTED;
+  const int rows = experts + (shared_gate_w ? 1 : 0), ldz = experts + 1;
+  const dim3 grid((unsigned)((tokens + RT - 1) / RT), (unsigned)((rows + 3) / 4));
   DINFER_DISPATCH_DTYPE(dtype, {
-    moe_route_kernel<S><<<(unsigned)tokens, 256, 0, stream>>>((const S*)x, ld_x, router, shared_gate_w, experts, top,
-                                                             width, idx, share, shared_gate);
+    moe_logits_kernel<S><<<grid, 256, 0, stream>>>((const S*)x, ld_x, (int)tokens, router, shared_gate_w, experts, width,
+                                                   z, ldz);
   });
+  if (launch_status() != OK) return ERR_LAUNCH;
+  moe_topk_kernel<<<(unsigned)((tokens + 3) / 4), 256, 0, stream>>>(z, ldz, (int)tokens, experts, top,
+                                                                   shared_gate_w ? 1 : 0, idx, share, shared_gate);
   return launch_status();
 }
 
-extern "C" int dinfer_moe_scatter(const int32_t* idx, int64_t entries, int experts, int32_t* offsets, int32_t* perm,
-                                  int32_t* tiles, int64_t max_tiles, hipStream_t stream) {
+extern "C" int dinfer_moe_scatter(const int32_t* idx, int64_t entries, int experts, int tile_rows, int32_t* offsets,
+                                  int32_t* perm, int32_t* tiles, int64_t max_tiles, hipStream_t stream) {
   if (entries <= 0) return OK;
-  if (experts <= 0 || entries > 0x7fffffff || max_tiles < (entries + BM - 1) / BM + experts) return ERR_BAD_SHAPE;
+  if (experts <= 0 || tile_rows <= 0 || entries > 0x7fffffff ||
+      max_tiles < (entries + tile_rows - 1) / tile_rows + experts)
+    return ERR_BAD_SHAPE;
   if (experts > MAX_EXPERTS) return ERR_UNSUPPORTED;
-  moe_scatter_kernel<<<1, 1024, 0, stream>>>(idx, (int)entries, experts, BM, offsets, perm, tiles, (int)max_tiles);
+  moe_scatter_kernel<<<1, 1024, 0, stream>>>(idx, (int)entries, experts, tile_rows, offsets, perm, tiles, (int)max_tiles);
   return launch_status();
 }
 
@@ -400,6 +548,13 @@ extern "C" int dinfer_moe_combine(int dtype, const void* y, int64_t ld_y, const 
                                   int width, hipStream_t stream) {
   if (tokens <= 0) return OK;
   if (top <= 0 || width <= 0 || tokens > 0x7fffffff) return ERR_BAD_SHAPE;
+  const bool vec = dtype == DT_BF16 && width % 8 == 0 && ld_y % 8 == 0 && ld_o % 8 == 0 && (!shared || ld_s % 8 == 0) &&
+                   ((uintptr_t)y % 16) == 0 && ((uintptr_t)out % 16) == 0 && ((uintptr_t)shared % 16) == 0;
+  if (vec) {
+    moe_combine_bf16x8_kernel<<<(unsigned)tokens, width >= 2048 ? 256 : 64, 0, stream>>>(
+        (const bf16*)y, ld_y, share, top, (const bf16*)shared, ld_s, shared_gate, (bf16*)out, ld_o, width);
+    return launch_status();
+  }
   DINFER_DISPATCH_DTYPE(dtype, {
     moe_combine_kernel<S><<<(unsigned)tokens, 256, 0, stream>>>((const S*)y, ld_y, share, top, (const S*)shared, ld_s,
                                                                shared_gate, (S*)out, ld_o, width);

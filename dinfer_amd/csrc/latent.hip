@@ -197,7 +197,7 @@ __global__ void __launch_bounds__(256) latent_attn_mfma_kernel(
     int64_t max_blocks, const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ seq_lens, int num_reqs,
     float scale_log2, int window, int H, int R, int dr, int page, int splits) {
   constexpr int NC = NT / 2 + 4;
-  extern __shared__ float meet[];   // [16][R + 2]: one wave's output, max and sum on their way to wave 0
+  extern __shared__ float meet[];   // [16][R + 4]: one wave's output, max and sum on their way to wave 0
   // which request and which of its row tiles
   int tile = blockIdx.x, b = 0, q_len = 0;
   for (; b < num_reqs; ++b) {
@@ -312,7 +312,7 @@ __global__ void __launch_bounds__(256) latent_attn_mfma_kernel(
   l += __shfl_xor(l, 32, 64);
 
   // the waves meet: one after the other hands its state to wave 0
-  const int ldm = R + 2;
+  const int ldm = R + 4;
   for (int w = 1; w < 4; ++w) {
     if (wave == w) {
 #pragma unroll
@@ -361,28 +361,44 @@ __global__ void __launch_bounds__(256) latent_attn_mfma_kernel(
   }
 }
 
-// One workgroup per (token, head) row: the parts' (max, sum, output) become the row's output.
+// One workgroup per (token, head) row: the parts' (max, sum, output) become the row's output. A part is R + 4 floats
+// (output, max, sum, two unused), so its rows are read 16 bytes a lane.
 __global__ void __launch_bounds__(128) latent_attn_merge_kernel(const float* __restrict__ part, bf16* __restrict__ out,
                                                                 int64_t ld_out, int H, int R, int splits) {
+  __shared__ float wgt[256];
+  __shared__ float inv_s;
   const int64_t row = blockIdx.x;
-  const int ldm = R + 2;
+  const int ldm = R + 4;
   const float* pr = part + row * splits * (int64_t)ldm;
-  float mt = -INFINITY;
-  for (int s = 0; s < splits; ++s) mt = fmaxf(mt, pr[s * (int64_t)ldm + R]);
-  float lt = 0.f;
-  for (int s = 0; s < splits; ++s) {
-    const float ms = pr[s * (int64_t)ldm + R];
-    if (ms != -INFINITY) lt += pr[s * (int64_t)ldm + R + 1] * exp2_of(ms - mt);
-  }
-  const float inv = lt > 0.f ? 1.f / lt : 0.f;
-  bf16* orow = out + (row / H) * ld_out + (row % H) * (int64_t)R;
-  for (int d = threadIdx.x; d < R; d += blockDim.x) {
-    float acc = 0.f;
-    for (int s = 0; s < splits; ++s) {
+  if (threadIdx.x < 64) {     // the first wave: the weights of the parts
+    float mt = -INFINITY;
+    for (int s = threadIdx.x; s < splits; s += 64) mt = fmaxf(mt, pr[s * (int64_t)ldm + R]);
+    mt = wave_max(mt);
+    float lt = 0.f;
+    for (int s = threadIdx.x; s < splits; s += 64) {
       const float ms = pr[s * (int64_t)ldm + R];
-      if (ms != -INFINITY) acc += pr[s * (int64_t)ldm + d] * exp2_of(ms - mt);
+      const float w = ms == -INFINITY ? 0.f : exp2_of(ms - mt);
+      wgt[s] = w;
+      lt += w * pr[s * (int64_t)ldm + R + 1];
     }
-    orow[d] = (bf16)(acc * inv);
+    lt = wave_sum(lt);
+    if (threadIdx.x == 0) inv_s = lt > 0.f ? 1.f / lt : 0.f;
+  }
+  __syncthreads();
+  const float inv = inv_s;
+  bf16* orow = out + (row / H) * ld_out + (row % H) * (int64_t)R;
+  for (int d = threadIdx.x * 4; d < R; d += 128 * 4) {
+    f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int s = 0; s < splits; ++s) {
+      const f32x4 v = *(const f32x4*)(pr + s * (int64_t)ldm + d);
+      const float w = wgt[s];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) acc[i] = fmaf(w, v[i], acc[i]);
+    }
+    bf16x4 y;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) y[i] = (bf16)(acc[i] * inv);
+    *(bf16x4*)(orow + d) = y;
   }
 }
 
@@ -433,7 +449,7 @@ extern "C" int dinfer_latent_mfma_supports(int R, int dr, int page_size) {
 }
 
 // bf16. cache [blocks, page, R + dr] and cache_t [blocks, R, page]. splits > 1: every request brings one row; part holds
-// tokens * heads * splits * (R + 2) floats.
+// tokens * heads * splits * (R + 4) floats.
 extern "C" int dinfer_latent_attn_mfma(const void* qa, int64_t ld_qa, void* out, int64_t ld_out, float* part,
                                        int64_t part_floats, const void* cache, const void* cache_t,
                                        const int32_t* block_table, int64_t max_blocks, const int32_t* cu_seqlens,
@@ -444,12 +460,12 @@ extern "C" int dinfer_latent_attn_mfma(const void* qa, int64_t ld_qa, void* out,
       ((uintptr_t)qa % 16) || ((uintptr_t)out % 8) || ((uintptr_t)cache % 16) || ((uintptr_t)cache_t % 8))
     return ERR_BAD_SHAPE;
   if (!dinfer_latent_mfma_supports(R, dr, page_size)) return ERR_UNSUPPORTED;
-  if (splits > 1 && (tokens != num_reqs || !part || part_floats < tokens * heads * splits * (int64_t)(R + 2)))
+  if (splits > 1 && (tokens != num_reqs || !part || part_floats < tokens * heads * splits * (int64_t)(R + 4) || splits > 256))
     return ERR_WORKSPACE;
   const int64_t tiles = (tokens * heads + 15) / 16 + num_reqs;
   if (tiles > 0x7fffffff || splits > 65535) return ERR_UNSUPPORTED;
   const dim3 grid((unsigned)tiles, (unsigned)splits);
-  const size_t lds = (size_t)16 * (R + 2) * sizeof(float);
+  const size_t lds = (size_t)16 * (R + 4) * sizeof(float);
   const float sl = scale * LOG2E;
 #define LAUNCH(NT)                                                                                                     \
   latent_attn_mfma_kernel<NT><<<grid, 256, lds, stream>>>((const bf16*)qa, ld_qa, (bf16*)out, ld_out, part,           \

@@ -12,7 +12,7 @@ from . import ops
 
 TARGET_WORKGROUPS = 512
 MAX_SPLITS = 64
-SHORTEST_PART = 128
+SHORTEST_PART = 512    # keys of the longest request in one part (its four waves take a quarter each), at least
 
 
 class Workspace:
@@ -26,7 +26,7 @@ class Workspace:
         self.part = None
         if self.mfma:
             units = max(self.splits(n) * n for n in range(1, ctx.max_reqs + 1)) * heads
-            self.part = ctx.workspace.buffer("latent_partials", units * (rank + 2), dtype=torch.float32, rows=1)
+            self.part = ctx.workspace.buffer("latent_partials", units * (rank + 4), dtype=torch.float32, rows=1)
 
     def splits(self, num_reqs: int) -> int:
         """Parts per request in a step of single rows: a function of the batch size only, so a captured graph stays valid."""

@@ -32,10 +32,10 @@ SIGNATURES = {
     "dinfer_latent_attn_mfma": ("latent", [_P, _L, _P, _L, _P, _L, _P, _P, _P, _L, _P, _P, _I, _L, _F, _I, _I, _I, _I, _I, _I, _P]),
     "dinfer_latent_attn_ref": ("latent", [_I, _P, _L, _P, _L, _P, _P, _L, _P, _P, _I, _L, _F, _I, _I, _I, _I, _I, _P]),
     "dinfer_heads_nt": ("grouped", [_I, _P, _L, _L, _P, _L, _L, _P, _L, _L, _L, _L, _L, _L, _P, _L, _P]),
-    "dinfer_experts_nt": ("grouped", [_I, _I, _P, _L, _P, _L, _L, _P, _L, _L, _L, _P, _L, _P, _P, _I, _I, _P]),
-    "dinfer_moe_tile_rows": ("grouped", []),
-    "dinfer_moe_route": ("grouped", [_I, _P, _L, _L, _P, _P, _I, _I, _I, _P, _P, _P, _P]),
-    "dinfer_moe_scatter": ("grouped", [_P, _L, _I, _P, _P, _P, _L, _P]),
+    "dinfer_experts_nt": ("grouped", [_I, _I, _P, _L, _P, _L, _L, _P, _L, _L, _L, _P, _L, _I, _P, _P, _I, _I, _P]),
+    "dinfer_moe_tile_rows": ("grouped", [_I, _L, _I, _L, _L]),
+    "dinfer_moe_route": ("grouped", [_I, _P, _L, _L, _P, _P, _I, _I, _I, _P, _P, _P, _P, _P]),
+    "dinfer_moe_scatter": ("grouped", [_P, _L, _I, _I, _P, _P, _P, _L, _P]),
     "dinfer_moe_combine": ("grouped", [_I, _P, _L, _P, _I, _P, _L, _P, _P, _L, _L, _I, _P]),
     "dinfer_rmsnorm": ("norm", [_I, _P, _P, _P, _P, _I, _P, _L, _L, _L, _L, _F, _F, _P]),
     "dinfer_qkv_post": (

@@ -266,7 +266,7 @@ def latent_attn_mfma(qa: torch.Tensor, out: torch.Tensor, cache: torch.Tensor, c
                      rank: int, rot_dim: int, page_size: int) -> torch.Tensor:
     """latent_attn_ref on the matrix cores (bfloat16): cache_t [blocks, rank, page] holds the latents once more, the
     pages transposed. splits > 1 (steps in which every request brings one row): each request's keys are cut into that
-    many parts on the device and merged; part: float32 scratch of tokens * heads * splits * (rank + 2)."""
+    many parts on the device and merged; part: float32 scratch of tokens * heads * splits * (rank + 4)."""
     _need_gpu(qa, out, cache, cache_t, block_table, cu_seqlens, seq_lens, part)
     _check_latent(qa, out, cache, block_table, cu_seqlens, seq_lens, num_reqs, tokens, heads, rank, rot_dim, page_size)
     assert qa.dtype == torch.bfloat16 and cache_t.dtype == torch.bfloat16 and cache_t.is_contiguous()
@@ -303,59 +303,65 @@ MOE_MAX_EXPERTS = 1024   # the routing and sorting kernels keep one number an ex
 MOE_MAX_TOP = 64         # a lane of the routing wave keeps one choice
 
 
-def moe_tile_rows() -> int:
-    return int(lib.get("dinfer_moe_tile_rows")())
+def moe_tile_rows(dtype: torch.dtype, entries: int, experts: int, k_in: int, k_mid: int) -> int:
+    """Rows of a row tile for the two products of a routed layer over `entries` (token, choice) pairs: what the kernel
+    that will run them takes (16 where an expert gets few rows, 128 for many, 64 on the vector ALUs)."""
+    return int(lib.get("dinfer_moe_tile_rows")(dtype_code(dtype), entries, experts, k_in, k_mid))
 
 
-def moe_max_tiles(entries: int, experts: int) -> int:
+def moe_max_tiles(entries: int, experts: int, tile_rows: int) -> int:
     """Length of the work list for `entries` (token, choice) pairs: every expert may end with a tile that is not full."""
-    return -(-entries // moe_tile_rows()) + experts
+    return -(-entries // tile_rows) + experts
 
 
 def moe_route(x: torch.Tensor, router: torch.Tensor, shared_gate_w: torch.Tensor | None, idx: torch.Tensor,
-              share: torch.Tensor, shared_gate: torch.Tensor | None, tokens: int, top: int) -> None:
+              share: torch.Tensor, shared_gate: torch.Tensor | None, tokens: int, top: int, z: torch.Tensor) -> None:
     """Per token: logits x @ router.T in float (router float32 [experts, width]), idx[t] the `top` largest (lowest index
-    among equals), share[t] the softmax over them; shared_gate[t] = sigmoid(x . shared_gate_w) where that is given."""
-    _need_gpu(x, router, shared_gate_w, idx, share, shared_gate)
+    among equals), share[t] the softmax over them; shared_gate[t] = sigmoid(x . shared_gate_w) where that is given.
+    z: float32 scratch of tokens * (experts + 1) for the logits."""
+    _need_gpu(x, router, shared_gate_w, idx, share, shared_gate, z)
     experts, width = router.shape
     assert router.dtype == torch.float32 and router.is_contiguous() and x.shape[1] == width and x.shape[0] >= tokens
     assert idx.dtype == torch.int32 and share.dtype == torch.float32 and idx.is_contiguous() and share.is_contiguous()
     assert idx.numel() >= tokens * top and share.numel() >= tokens * top
+    assert z.dtype == torch.float32 and z.is_contiguous() and z.numel() >= tokens * (experts + 1)
     if shared_gate_w is not None:
         assert shared_gate_w.dtype == torch.float32 and shared_gate_w.numel() == width and shared_gate_w.is_contiguous()
         assert shared_gate is not None and shared_gate.dtype == torch.float32 and shared_gate.numel() >= tokens
     lib.call("dinfer_moe_route", dtype_code(x.dtype), x.data_ptr(), _rows(x), tokens, router.data_ptr(),
-             _ptr(shared_gate_w), experts, top, width, idx.data_ptr(), share.data_ptr(),
+             _ptr(shared_gate_w), experts, top, width, z.data_ptr(), idx.data_ptr(), share.data_ptr(),
              _ptr(shared_gate) if shared_gate_w is not None else 0, _stream())
 
 
 def moe_scatter(idx: torch.Tensor, entries: int, experts: int, offsets: torch.Tensor, perm: torch.Tensor,
-                tiles: torch.Tensor) -> None:
+                tiles: torch.Tensor, tile_rows: int) -> None:
     """Sorts the entries (token * top + choice) by expert: offsets [experts + 1], perm [entries] (sorted place -> entry),
     tiles [n, 2] the work list of experts_nt ((expert, first sorted place) per row tile, -1 beyond the last)."""
     _need_gpu(idx, offsets, perm, tiles)
     assert idx.dtype == offsets.dtype == perm.dtype == tiles.dtype == torch.int32
     assert idx.numel() >= entries and perm.numel() >= entries and offsets.numel() >= experts + 1
     assert tiles.is_contiguous() and tiles.dim() == 2 and tiles.shape[1] == 2
-    n = moe_max_tiles(entries, experts)
+    n = moe_max_tiles(entries, experts, tile_rows)
     assert tiles.shape[0] >= n
-    lib.call("dinfer_moe_scatter", idx.data_ptr(), entries, experts, offsets.data_ptr(), perm.data_ptr(),
+    lib.call("dinfer_moe_scatter", idx.data_ptr(), entries, experts, tile_rows, offsets.data_ptr(), perm.data_ptr(),
              tiles.data_ptr(), n, _stream())
 
 
 def experts_nt(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, entries: int, tiles: torch.Tensor,
-               offsets: torch.Tensor, perm: torch.Tensor, *, gated: bool, a_div: int, c_to_perm: bool) -> torch.Tensor:
+               offsets: torch.Tensor, perm: torch.Tensor, *, gated: bool, a_div: int, c_to_perm: bool,
+               tile_rows: int) -> torch.Tensor:
     """The products of all experts in one launch. w [experts, rows, K]; gated: rows = 2 N, gate rows first, and
     out = silu(a Wg^T) * (a Wu^T). a_div > 0: the row of sorted place i is a[perm[i] // a_div] (the step's tokens),
-    0: a[i]. c_to_perm: the result of sorted place i goes to out[perm[i]], else to out[i]."""
+    0: a[i]. c_to_perm: the result of sorted place i goes to out[perm[i]], else to out[i]. tile_rows: what moe_scatter
+    made the work list with."""
     _need_gpu(a, w, out, tiles, offsets, perm)
     experts, rows, k = w.shape
     n = rows // 2 if gated else rows
     assert w.is_contiguous() and a.dtype == w.dtype == out.dtype and a.shape[1] == k and out.shape[1] == n
     assert out.shape[0] >= entries and (a_div > 0 or a.shape[0] >= entries)
     lib.call("dinfer_experts_nt", dtype_code(a.dtype), 1 if gated else 0, a.data_ptr(), _rows(a), w.data_ptr(), k,
-             rows * k, out.data_ptr(), _rows(out), n, k, tiles.data_ptr(), moe_max_tiles(entries, experts),
-             offsets.data_ptr(), perm.data_ptr(), int(a_div), 1 if c_to_perm else 0, _stream())
+             rows * k, out.data_ptr(), _rows(out), n, k, tiles.data_ptr(), moe_max_tiles(entries, experts, tile_rows),
+             int(tile_rows), offsets.data_ptr(), perm.data_ptr(), int(a_div), 1 if c_to_perm else 0, _stream())
     return out
 
 

@@ -70,10 +70,12 @@ class RoutedExperts(FeedForward):
         i32 = torch.int32
         self.idx = torch.zeros(n, dtype=i32, device=dev)
         self.share = torch.zeros(n, dtype=torch.float32, device=dev)
+        self.logits = torch.zeros(ctx.max_tokens * (self.experts + 1), dtype=torch.float32, device=dev)
         self.shared_gate = torch.zeros(ctx.max_tokens, dtype=torch.float32, device=dev)
         self.offsets = torch.zeros(self.experts + 1, dtype=i32, device=dev)
         self.perm = torch.zeros(n, dtype=i32, device=dev)
-        self.tiles = torch.zeros((ops.moe_max_tiles(n, self.experts), 2), dtype=i32, device=dev)
+        self.dtype = ctx.dtype
+        self.tiles = torch.zeros((ops.moe_max_tiles(n, self.experts, 16), 2), dtype=i32, device=dev)   # the smallest tile: the longest list
         self.act_buf = ws.buffer("moe_act", self.intermediate, rows=n)
         self.y_buf = ws.buffer("moe_y", self.hidden, rows=n)
         self.out_buf = ws.buffer("ffn_out", self.hidden)
@@ -83,11 +85,12 @@ class RoutedExperts(FeedForward):
     def forward(self, x, batch, into=None):
         T, top = batch.num_tokens, self.top
         n = T * top
-        ops.moe_route(x, self.router, self.sg, self.idx, self.share, self.shared_gate, T, top)
-        ops.moe_scatter(self.idx, n, self.experts, self.offsets, self.perm, self.tiles)
+        ops.moe_route(x, self.router, self.sg, self.idx, self.share, self.shared_gate, T, top, self.logits)
+        rows = ops.moe_tile_rows(self.dtype, n, self.experts, self.hidden, self.intermediate)   # follows the step's count alone
+        ops.moe_scatter(self.idx, n, self.experts, self.offsets, self.perm, self.tiles, rows)
         ops.experts_nt(x, self.w_in, self.act_buf, n, self.tiles, self.offsets, self.perm, gated=True, a_div=top,
-                       c_to_perm=False)
+                       c_to_perm=False, tile_rows=rows)
         ops.experts_nt(self.act_buf, self.w_out, self.y_buf, n, self.tiles, self.offsets, self.perm, gated=False, a_div=0,
-                       c_to_perm=True)
+                       c_to_perm=True, tile_rows=rows)
         shared = self.shared.forward(x, batch) if self.shared is not None else None
         return ops.moe_combine(self.y_buf, self.share, top, shared, self.shared_gate, self.out_buf, T)

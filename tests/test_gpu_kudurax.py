@@ -491,7 +491,7 @@ def test_latent_attention_kernels(case_no, kernel):
         assert ops.latent_mfma_supports(R, dr, page)
         cache_t = dev["cache"][:, :, :R].transpose(1, 2).contiguous()
         splits = 5 if kernel == "mfma_split" else 1
-        part = torch.zeros(T * H * splits * (R + 2), dtype=torch.float32, device="cuda")
+        part = torch.zeros(T * H * splits * (R + 4), dtype=torch.float32, device="cuda")
         ops.latent_attn_mfma(dev["qa"], out, dev["cache"], cache_t, dev["bt"], dev["cu"], dev["seq"], B, T, splits, part, **geo)
     got = out.double().cpu()
     tol = 2e-5 if dtype == torch.float32 else 0.03
