@@ -291,10 +291,9 @@ __global__ void __launch_bounds__(256) grouped_mfma_small_kernel(Groups p) {
 constexpr int MAX_EXPERTS = 1024;
 
 // Router logits: a wave takes one expert (the row after the last expert is the shared expert's gate vector) and up to
-// RT tokens, so a router row is read once per RT tokens; a lane sums every 64th entry, then the lanes meet. z [T, ldz].
-constexpr int RT = 8;
-
-template <class S>
+// RT tokens (8 in steps of many tokens, so that a router row is read once per 8; 1 in steps of few, where more
+// workgroups matter more); a lane sums every 64th entry, then the lanes meet. z [T, ldz].
+template <class S, int RT>
 __global__ void __launch_bounds__(256) moe_logits_kernel(const S* __restrict__ x, int64_t ld_x, int tokens,
                                                          const float* __restrict__ wr, const float* __restrict__ wsg,
                                                          int E, int width, float* __restrict__ z, int ldz) {
@@ -521,10 +520,15 @@ extern "C" int dinfer_moe_route(int dtype, const void* x, int64_t ld_x, int64_t 
   if (experts <= 0 || top <= 0 || top > experts || width <= 0 || tokens > 0x7fffffff || !z) return ERR_BAD_SHAPE;
   if (experts > MAX_EXPERTS || top > 64) return ERR_UNSUPPORTED;
   const int rows = experts + (shared_gate_w ? 1 : 0), ldz = experts + 1;
-  const dim3 grid((unsigned)((tokens + RT - 1) / RT), (unsigned)((rows + 3) / 4));
+  const int rt = tokens <= 128 ? 1 : 8;
+  const dim3 grid((unsigned)((tokens + rt - 1) / rt), (unsigned)((rows + 3) / 4));
   DINFER_DISPATCH_DTYPE(dtype, {
-    moe_logits_kernel<S><<<grid, 256, 0, stream>>>((const S*)x, ld_x, (int)tokens, router, shared_gate_w, experts, width,
-                                                   z, ldz);
+    if (rt == 1)
+      moe_logits_kernel<S, 1><<<grid, 256, 0, stream>>>((const S*)x, ld_x, (int)tokens, router, shared_gate_w, experts,
+                                                        width, z, ldz);
+    else
+      moe_logits_kernel<S, 8><<<grid, 256, 0, stream>>>((const S*)x, ld_x, (int)tokens, router, shared_gate_w, experts,
+                                                        width, z, ldz);
   });
   if (launch_status() != OK) return ERR_LAUNCH;
   moe_topk_kernel<<<(unsigned)((tokens + 3) / 4), 256, 0, stream>>>(z, ldz, (int)tokens, experts, top,

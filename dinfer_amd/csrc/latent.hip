@@ -185,28 +185,47 @@ __device__ __forceinline__ float exp2_of(float x) { return __builtin_amdgcn_exp2
 // entries (dr <= 128). v_mfma_f32_16x16x32_bf16: lane l holds row (first operand) or column (second) l % 16 and the 8
 // entries of the contraction that belong to group l / 16; of the result, column l % 16 and rows 4 (l / 16) .. + 3.
 //   scores   first operand 16 keys x 32 key entries (rows of the cache, 16 bytes a lane), second the queries;
-//            lane l gets, for query row l % 16, the keys 4 (l / 16) .. + 3 of each of the block's two key tiles
-//   values   contraction over the block's 32 keys in the order (group g: keys 4g .. 4g+3 of the first tile, then of the
-//            second), which is the order in which a lane holds its weights; first operand 16 latent entries x those keys
-//            (two 8-byte pieces of the transposed pages), second the weights; the result is O^T: lane l holds query
-//            row l % 16 and latent entries 16 tile + 4 (l / 16) .. + 3.
-template <int NT>
+//            lane l gets, for query row l % 16, rows 4 (l / 16) .. + 3 of each of the block's two key tiles
+//   values   contraction over the block's 32 keys in the order in which a lane holds its weights, which the rows of the
+//            two key tiles are numbered for (see the loop): group g holds keys 8g .. 8g+7; first operand 16 latent
+//            entries x those keys (16 bytes of a transposed page), second the weights; the result is O^T: lane l holds
+//            query row l % 16 and latent entries 16 tile + 4 (l / 16) .. + 3.
+// SOLO: steps with prompt portions: every wave takes a row tile of its own and walks all its keys (the four waves of
+// a workgroup take consecutive tiles, so they ask for the same keys at about the same time and meet in the cache);
+// otherwise (steps of single rows) the four waves share one row tile and deal its keys among themselves.
+template <int NT, bool SOLO>
 __global__ void __launch_bounds__(256) latent_attn_mfma_kernel(
     const bf16* __restrict__ qa, int64_t ld_qa, bf16* __restrict__ out, int64_t ld_out, float* __restrict__ part,
     const bf16* __restrict__ cache, const bf16* __restrict__ cache_t, const int32_t* __restrict__ block_table,
     int64_t max_blocks, const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ seq_lens, int num_reqs,
     float scale_log2, int window, int H, int R, int dr, int page, int splits) {
   constexpr int NC = NT / 2 + 4;
+  constexpr int KG = 4, VG = NT < 8 ? NT : 8;   // loads of keys (x 2 tiles) and of values in flight before a product waits (more cost registers and with them the second wave of a SIMD: measured slower)
   extern __shared__ float meet[];   // [16][R + 4]: one wave's output, max and sum on their way to wave 0
-  // which request and which of its row tiles
-  int tile = blockIdx.x, b = 0, q_len = 0;
-  for (; b < num_reqs; ++b) {
-    q_len = cu_seqlens[b + 1] - cu_seqlens[b];
-    const int tiles = (q_len * H + 15) >> 4;
-    if (tile < tiles) break;
-    tile -= tiles;
+  // which request and which of its row tiles: 64 requests at a time, one a lane, counted with a prefix sum over the wave
+  int tile = SOLO ? blockIdx.x * 4 + (int)(threadIdx.x >> 6) : blockIdx.x, b = -1, q_len = 0;
+  {
+    const int ln = threadIdx.x & 63;
+    for (int b0 = 0; b0 < num_reqs && b < 0; b0 += 64) {
+      const int mine = b0 + ln < num_reqs ? cu_seqlens[b0 + ln + 1] - cu_seqlens[b0 + ln] : 0;
+      int upto = (mine * H + 15) >> 4;      // tiles of the requests b0 .. b0 + ln
+#pragma unroll
+      for (int o = 1; o < 64; o <<= 1) {
+        const int v = __shfl_up(upto, o, 64);
+        if (ln >= o) upto += v;
+      }
+      const unsigned long long holds = __ballot(tile < upto);
+      if (holds) {
+        const int at = __ffsll((long long)holds) - 1;
+        b = b0 + at;
+        q_len = __shfl(mine, at, 64);
+        tile -= at ? __shfl(upto, at - 1, 64) : 0;
+      } else {
+        tile -= __shfl(upto, 63, 64);
+      }
+    }
   }
-  if (b >= num_reqs) return;   // (the whole workgroup)
+  if (b < 0) return;   // (SOLO: this wave, and no barrier follows; else the whole workgroup: every wave counts the same)
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, lr = lane & 15, g = lane >> 4;
   const int DK = R + dr;
   const int start = seq_lens[b] - q_len;
@@ -220,7 +239,7 @@ __global__ void __launch_bounds__(256) latent_attn_mfma_kernel(
   const int lowest = window > 0 ? (p - window + 1 > 0 ? p - window + 1 : 0) : 0;   // of this lane's row
   const int kb0 = first & ~31;
   const int nblk = (p_last - kb0) / 32 + 1;
-  const int parts = splits * 4, me = blockIdx.y * 4 + wave;
+  const int parts = SOLO ? 1 : splits * 4, me = SOLO ? 0 : blockIdx.y * 4 + wave;
   const int per = (nblk + parts - 1) / parts;
   const int blk_lo = me * per, blk_hi = blk_lo + per < nblk ? blk_lo + per : nblk;
   const int32_t* bt = block_table + (int64_t)b * max_blocks;
@@ -242,30 +261,53 @@ __global__ void __launch_bounds__(256) latent_attn_mfma_kernel(
   for (int t = 0; t < NT; ++t) o[t] = f32x4{0.f, 0.f, 0.f, 0.f};
   float m = -INFINITY, l = 0.f;
 
+  // Row r of key tile t stands for key kb + 8 (r / 4) + 4 t + r % 4, so that the eight weights a lane holds after the
+  // scores (rows 4g .. 4g+3 of both tiles) belong to the eight consecutive keys kb + 8g .. + 7: its operand of the
+  // product with the values is 16 bytes of a transposed page.
+  const int kofs = 8 * (lr >> 2) + (lr & 3);
   for (int blk = blk_lo; blk < blk_hi; ++blk) {
     const int kb = kb0 + blk * 32;
-    f32x4 s[2];
+    const bf16* krow[2];
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
-      int key = kb + 16 * t + lr;
+      int key = kb + kofs + 4 * t;
       key = key < first ? first : (key > p_last ? p_last : key);   // a row that exists; what lies outside is masked below
-      const bf16* krow = cache + ((int64_t)bt[key / page] * page + (key % page)) * DK + 8 * g;
-      f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+      krow[t] = cache + ((int64_t)bt[key / page] * page + (key % page)) * DK;
+    }
+    const bf16* vrow;
+    {
+      int key = kb + 8 * g;
+      const int lo8 = first & ~7, hi8 = p_last & ~7;
+      key = key < lo8 ? lo8 : (key > hi8 ? hi8 : key);
+      vrow = cache_t + (int64_t)bt[key / page] * R * page + (key % page);
+    }
+    f32x4 s[2] = {f32x4{0.f, 0.f, 0.f, 0.f}, f32x4{0.f, 0.f, 0.f, 0.f}};
+    // loads in groups, so that several are in flight before the first product waits
 #pragma unroll
-      for (int c = 0; c < NC; ++c) {
-        if (32 * c < DK) {
-          const bf16x8 a = (32 * c + 8 * g < DK) ? *(const bf16x8*)(krow + 32 * c) : zero;
-          acc = mfma16(a, qf[c], acc);
+    for (int c0 = 0; c0 < NC; c0 += KG) {
+      if (32 * c0 < DK) {
+        bf16x8 ka[2][KG];
+#pragma unroll
+        for (int j = 0; j < KG; ++j) {
+          // entries beyond the row meet zeros of the query; the address stays inside the row
+          const int d = 32 * (c0 + j) + 8 * g;
+          const int dc = d < DK ? d : 0;
+#pragma unroll
+          for (int t = 0; t < 2; ++t) ka[t][j] = *(const bf16x8*)(krow[t] + dc);
         }
+#pragma unroll
+        for (int j = 0; j < KG; ++j)
+#pragma unroll
+          for (int t = 0; t < 2; ++t)
+            if (c0 + j < NC) s[t] = mfma16(ka[t][j], qf[c0 + j < NC ? c0 + j : 0], s[t]);
       }
-      s[t] = acc;
     }
     float mx = -INFINITY;
 #pragma unroll
     for (int t = 0; t < 2; ++t)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const int key = kb + 16 * t + 4 * g + i;
+        const int key = kb + 8 * g + 4 * t + i;
         const float v = (key <= p && key >= lowest) ? s[t][i] * scale_log2 : -INFINITY;
         s[t][i] = v;
         mx = fmaxf(mx, v);
@@ -286,25 +328,18 @@ __global__ void __launch_bounds__(256) latent_attn_mfma_kernel(
       }
     l = l * alpha + psum;   // this lane's share of the row's sum; the four shares meet after the walk
     m = m_new;
-    // the latents of keys kb + 4g .. + 3 and kb + 16 + 4g .. + 3, one latent entry a lane
-    const bf16* vt[2];
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
-      int key = kb + 16 * t + 4 * g;
-      const int lo4 = first & ~3, hi4 = p_last & ~3;
-      key = key < lo4 ? lo4 : (key > hi4 ? hi4 : key);
-      vt[t] = cache_t + (int64_t)bt[key / page] * R * page + (key % page);
-    }
+    for (int t0 = 0; t0 < NT; t0 += VG) {
+      if (16 * t0 < R) {
+        bf16x8 va[VG];
 #pragma unroll
-    for (int t = 0; t < NT; ++t) {
-      if (16 * t < R) {
-        const int64_t d = 16 * t + lr;
-        const bf16x4 a0 = *(const bf16x4*)(vt[0] + d * page);
-        const bf16x4 a1 = *(const bf16x4*)(vt[1] + d * page);
-        bf16x8 a;
+        for (int j = 0; j < VG; ++j) {
+          const int d = 16 * (t0 + j) + lr;
+          va[j] = *(const bf16x8*)(vrow + (int64_t)(d < R ? d : 0) * page);
+        }
 #pragma unroll
-        for (int i = 0; i < 4; ++i) { a[i] = a0[i]; a[4 + i] = a1[i]; }
-        o[t] = mfma16(a, pb, o[t] * alpha);
+        for (int j = 0; j < VG; ++j)
+          if (t0 + j < NT && 16 * (t0 + j) < R) o[t0 + j] = mfma16(va[j], pb, o[t0 + j] * alpha);
       }
     }
   }
@@ -313,7 +348,7 @@ __global__ void __launch_bounds__(256) latent_attn_mfma_kernel(
 
   // the waves meet: one after the other hands its state to wave 0
   const int ldm = R + 4;
-  for (int w = 1; w < 4; ++w) {
+  for (int w = 1; w < (SOLO ? 1 : 4); ++w) {
     if (wave == w) {
 #pragma unroll
       for (int t = 0; t < NT; ++t)
@@ -337,9 +372,9 @@ __global__ void __launch_bounds__(256) latent_attn_mfma_kernel(
     }
     __syncthreads();
   }
-  if (wave != 0 || !rv) return;
+  if ((!SOLO && wave != 0) || !rv) return;
   const int64_t trow = cu_seqlens[b] + tok;
-  if (splits == 1) {
+  if (SOLO || splits == 1) {
     const float inv = l > 0.f ? 1.f / l : 0.f;
     bf16* orow = out + trow * ld_out + (int64_t)head * R;
 #pragma unroll
@@ -457,26 +492,29 @@ extern "C" int dinfer_latent_attn_mfma(const void* qa, int64_t ld_qa, void* out,
                                        int heads, int R, int dr, int page_size, int splits, hipStream_t stream) {
   if (tokens <= 0 || num_reqs <= 0) return OK;
   if (heads <= 0 || max_blocks <= 0 || window < 0 || tokens > 0x7fffffff || splits < 1 || ld_qa % 8 || ld_out % 4 ||
-      ((uintptr_t)qa % 16) || ((uintptr_t)out % 8) || ((uintptr_t)cache % 16) || ((uintptr_t)cache_t % 8))
+      ((uintptr_t)qa % 16) || ((uintptr_t)out % 8) || ((uintptr_t)cache % 16) || ((uintptr_t)cache_t % 16))
     return ERR_BAD_SHAPE;
   if (!dinfer_latent_mfma_supports(R, dr, page_size)) return ERR_UNSUPPORTED;
   if (splits > 1 && (tokens != num_reqs || !part || part_floats < tokens * heads * splits * (int64_t)(R + 4) || splits > 256))
     return ERR_WORKSPACE;
   const int64_t tiles = (tokens * heads + 15) / 16 + num_reqs;
   if (tiles > 0x7fffffff || splits > 65535) return ERR_UNSUPPORTED;
-  const dim3 grid((unsigned)tiles, (unsigned)splits);
-  const size_t lds = (size_t)16 * (R + 4) * sizeof(float);
+  const bool solo = tokens != num_reqs;      // some request brings more than one row
+  const dim3 grid((unsigned)(solo ? (tiles + 3) / 4 : tiles), (unsigned)(solo ? 1 : splits));
+  const size_t lds = solo ? 0 : (size_t)16 * (R + 4) * sizeof(float);
   const float sl = scale * LOG2E;
-#define LAUNCH(NT)                                                                                                     \
-  latent_attn_mfma_kernel<NT><<<grid, 256, lds, stream>>>((const bf16*)qa, ld_qa, (bf16*)out, ld_out, part,           \
-                                                          (const bf16*)cache, (const bf16*)cache_t, block_table,       \
-                                                          max_blocks, cu_seqlens, seq_lens, num_reqs, sl, window, heads, \
-                                                          R, dr, page_size, splits)
-  if (R <= 64) LAUNCH(4);
-  else if (R <= 128) LAUNCH(8);
-  else if (R <= 256) LAUNCH(16);
-  else LAUNCH(32);
+#define LAUNCH(NT, SOLO)                                                                                               \
+  latent_attn_mfma_kernel<NT, SOLO><<<grid, 256, lds, stream>>>(                                                       \
+      (const bf16*)qa, ld_qa, (bf16*)out, ld_out, part, (const bf16*)cache, (const bf16*)cache_t, block_table,        \
+      max_blocks, cu_seqlens, seq_lens, num_reqs, sl, window, heads, R, dr, page_size, solo ? 1 : splits)
+#define PICK(NT) do { if (solo) LAUNCH(NT, true); else LAUNCH(NT, false); } while (0)
+  if (R <= 64) PICK(4);
+  else if (R <= 128) PICK(8);
+  else if (R <= 256) PICK(16);
+  else PICK(32);
+#undef PICK
 #undef LAUNCH
+  if (solo) return launch_status();
   if (launch_status() != OK) return ERR_LAUNCH;
   if (splits > 1)
     latent_attn_merge_kernel<<<(unsigned)(tokens * heads), 128, 0, stream>>>(part, (bf16*)out, ld_out, heads, R, splits);

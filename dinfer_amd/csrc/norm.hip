@@ -152,6 +152,78 @@ __global__ void __launch_bounds__(256) layernorm_kernel(const void* __restrict__
   }
 }
 
+// The same for widths that are multiples of 8 up to 256 * 8 * ITERS: a thread keeps its 8-entry pieces in registers
+// between the passes (one read of the row, no LDS but for the two sums), and moves them 16 or 32 bytes at a time.
+template <class SX, class SR, class SO, int ITERS>
+__global__ void __launch_bounds__(256) layernorm_regs_kernel(const SX* __restrict__ x, SR* __restrict__ residual,
+                                                             const int32_t* __restrict__ rows,
+                                                             const float* __restrict__ w, const float* __restrict__ b,
+                                                             SO* __restrict__ out, int64_t width, int64_t ld_x,
+                                                             int64_t ld_res, float eps) {
+  __shared__ float red[16];
+  const int64_t r = blockIdx.x;
+  const int64_t src = rows ? (int64_t)rows[r] : r;
+  const SX* xr = x + src * ld_x;
+  SR* rr = residual ? residual + src * ld_res : nullptr;
+  const int n8 = (int)(width / 8);
+  float v[ITERS][8];
+  float sum = 0.f;
+#pragma unroll
+  for (int it = 0; it < ITERS; ++it) {
+    const int i = it * 256 + threadIdx.x;
+    if (i < n8) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) v[it][j] = to_f32(xr[(int64_t)i * 8 + j]);
+      if (rr) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const SR s = from_f32<SR>(v[it][j] + to_f32(rr[(int64_t)i * 8 + j]));
+          rr[(int64_t)i * 8 + j] = s;
+          v[it][j] = to_f32(s);
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j) sum += v[it][j];
+    }
+  }
+  const float mean = block_sum(sum, red) / (float)width;
+  float ss = 0.f;
+#pragma unroll
+  for (int it = 0; it < ITERS; ++it) {
+    const int i = it * 256 + threadIdx.x;
+    if (i < n8) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) ss = add_square(ss, v[it][j] - mean);
+    }
+  }
+  const float inv = 1.f / sqrtf(block_sum(ss, red) / (float)width + eps);
+  SO* o = out + r * width;
+#pragma unroll
+  for (int it = 0; it < ITERS; ++it) {
+    const int i = it * 256 + threadIdx.x;
+    if (i < n8) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int64_t c = (int64_t)i * 8 + j;
+        o[c] = from_f32<SO>((v[it][j] - mean) * inv * w[c] + (b ? b[c] : 0.f));
+      }
+    }
+  }
+}
+
+template <class SX, class SR, class SO>
+void launch_layernorm_regs(const void* x, void* residual, const int32_t* rows, const void* w, const void* b, void* out,
+                           int64_t n_rows, int64_t width, int64_t ld_x, int64_t ld_res, float eps, hipStream_t stream) {
+  const unsigned g = (unsigned)n_rows;
+#define LN(IT)                                                                                                        \
+  layernorm_regs_kernel<SX, SR, SO, IT><<<g, 256, 0, stream>>>((const SX*)x, (SR*)residual, rows, (const float*)w,    \
+                                                               (const float*)b, (SO*)out, width, ld_x, ld_res, eps)
+  if (width <= 256 * 8) LN(1);
+  else if (width <= 256 * 8 * 2) LN(2);
+  else LN(4);
+#undef LN
+}
+
 inline bool aligned16(const void* p) { return ((uintptr_t)p % 16) == 0; }
 
 }  // namespace
@@ -201,6 +273,23 @@ extern "C" int dinfer_layernorm(const void* x, int x_dtype, void* residual, int 
   if (width <= 0 || ld_x < width || (residual && ld_res < width) || n_rows > 0x7fffffff) return ERR_BAD_SHAPE;
   for (int dt : {x_dtype, res_dtype, param_dtype, out_dtype})
     if (dt != DT_F32 && dt != DT_BF16) return ERR_BAD_DTYPE;
+  // the combinations the engine meets, with float parameters, rows in registers: a float stream normed into the
+  // engine's type, alone or after a branch of the engine's type was added to it
+  if (param_dtype == DT_F32 && width % 8 == 0 && width <= 256 * 8 * 4 && ld_x % 8 == 0 && (!residual || ld_res % 8 == 0)) {
+    const bool res_f32 = !residual || res_dtype == DT_F32;
+    if (x_dtype == DT_F32 && res_f32 && out_dtype == DT_BF16) {
+      launch_layernorm_regs<float, float, bf16>(x, residual, rows, w, b, out, n_rows, width, ld_x, ld_res, eps, stream);
+      return launch_status();
+    }
+    if (x_dtype == DT_BF16 && res_f32 && out_dtype == DT_BF16) {
+      launch_layernorm_regs<bf16, float, bf16>(x, residual, rows, w, b, out, n_rows, width, ld_x, ld_res, eps, stream);
+      return launch_status();
+    }
+    if (x_dtype == DT_F32 && res_f32 && out_dtype == DT_F32) {
+      launch_layernorm_regs<float, float, float>(x, residual, rows, w, b, out, n_rows, width, ld_x, ld_res, eps, stream);
+      return launch_status();
+    }
+  }
   if (width > 16384) return ERR_UNSUPPORTED;
   layernorm_kernel<<<(unsigned)n_rows, 256, (size_t)width * sizeof(float), stream>>>(
       x, x_dtype, residual, res_dtype, rows, w, b, param_dtype, out, out_dtype, width, ld_x, ld_res, eps);
