@@ -152,12 +152,20 @@ __global__ void __launch_bounds__(256) grouped_valu_kernel(Groups p) {
 // memory in that order (16 bytes a lane).
 //
 // Many rows (tiles of 128): a workgroup takes 128 rows x 128 columns (gated: 64 columns of each half), its waves
-// 2 x 2, a wave 64 x 64: four row fragments and four column fragments feed sixteen MFMAs a step of 32 k.
+// 2 x 2, a wave 64 x 64. Both operands are staged through LDS 64 k at a time (16-byte pieces, read from memory by
+// the whole workgroup once, rows gathered through the tile's row list on the way), the next step's pieces are loaded
+// into registers while this step is multiplied; four row fragments and four column fragments feed sixteen MFMAs per
+// 32 k. Every output element is still summed over ascending k by one lane.
 constexpr int TM_BIG = 128, TM_SMALL = 16;
+
+constexpr int BIG_K = 64;            // k a step
+constexpr int BIG_LD = BIG_K + 8;    // row of a staged tile in LDS, padded: rows 16 bytes apart in the banks
 
 template <class O, bool GATED>
 __global__ void __launch_bounds__(256) grouped_mfma_big_kernel(Groups p) {
   __shared__ int64_t arow[TM_BIG];
+  __shared__ __attribute__((aligned(16))) bf16 As[TM_BIG * BIG_LD];
+  __shared__ __attribute__((aligned(16))) bf16 Ws[128 * BIG_LD];
   Tile tl;
   if (!tl.init(p)) return;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -168,42 +176,67 @@ __global__ void __launch_bounds__(256) grouped_mfma_big_kernel(Groups p) {
   const bf16* W = (const bf16*)p.W + (int64_t)tl.z * p.w_zs;
   if (threadIdx.x < TM_BIG) arow[threadIdx.x] = threadIdx.x < tl.rows ? tl.a_row(threadIdx.x) : -1;
   __syncthreads();
-  if (wm * 64 >= tl.rows) return;   // (no barrier follows)
-  const int lr = lane & 15, kq = lane >> 4;
-  const bf16* ap[4];
-  const bf16* wp[4];
+  // staging: a tile is 128 rows x 64 k = 1,024 pieces of 16 bytes, four a thread for each operand; piece q of a thread
+  // is row (q * 256 + thread) / 8, k piece (thread % 8)
+  const int sp = threadIdx.x & 7;
+  const bf16* ag[4];
+  const bf16* wg[4];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int64_t ar = arow[wm * 64 + i * 16 + lr];
-    ap[i] = ar >= 0 ? A + ar * p.lda + kq * 8 : nullptr;
-  }
-#pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    // gated: fragments 0, 1 are gate columns, 2, 3 the up columns of the same numbers
-    const int gn = GATED ? n0 + wn * 32 + (j & 1) * 16 + lr : n0 + wn * 64 + j * 16 + lr;
-    const int64_t wrow = GATED && j >= 2 ? gn + p.gate_n : gn;
-    wp[j] = gn < p.N ? W + wrow * p.ldw + kq * 8 : nullptr;
+  for (int q = 0; q < 4; ++q) {
+    const int row = (q * 256 + threadIdx.x) >> 3;
+    const int64_t ar = arow[row];
+    ag[q] = ar >= 0 ? A + ar * p.lda + sp * 8 : nullptr;
+    // row of the weight behind row `row` of the staged tile; gated: 64 gate rows, then the 64 up rows of the same numbers
+    const int gn = GATED ? n0 + (row & 63) : n0 + row;
+    const int64_t wrow = GATED && row >= 64 ? gn + p.gate_n : gn;
+    wg[q] = gn < p.N ? W + wrow * p.ldw + sp * 8 : nullptr;
   }
   bf16x8 zero;
 #pragma unroll
   for (int i = 0; i < 8; ++i) zero[i] = (bf16)0.f;
+  const int K = p.K;   // a multiple of 8 (checked on the host)
+  bf16x8 an[4], wn_[4];
+  auto fetch = [&](int k0) {
+    const bool in = k0 + sp * 8 < K;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      an[q] = (ag[q] && in) ? *(const bf16x8*)(ag[q] + k0) : zero;
+      wn_[q] = (wg[q] && in) ? *(const bf16x8*)(wg[q] + k0) : zero;
+    }
+  };
+  const int lr = lane & 15, kq = lane >> 4;
   f32x4 acc[4][4];
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
     for (int j = 0; j < 4; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
-  const int K = p.K;   // a multiple of 8 (checked on the host)
-  for (int k0 = 0; k0 < K; k0 += 32) {
-    const bool in = k0 + kq * 8 < K;
-    bf16x8 a[4], w[4];
+  fetch(0);
+  for (int k0 = 0; k0 < K; k0 += BIG_K) {
+    __syncthreads();      // the step before has read the tiles
 #pragma unroll
-    for (int i = 0; i < 4; ++i) a[i] = (ap[i] && in) ? *(const bf16x8*)(ap[i] + k0) : zero;
+    for (int q = 0; q < 4; ++q) {
+      const int row = (q * 256 + threadIdx.x) >> 3;
+      *(bf16x8*)(As + row * BIG_LD + sp * 8) = an[q];
+      *(bf16x8*)(Ws + row * BIG_LD + sp * 8) = wn_[q];
+    }
+    __syncthreads();
+    if (k0 + BIG_K < K) fetch(k0 + BIG_K);    // the next step's pieces travel while this one is multiplied
 #pragma unroll
-    for (int j = 0; j < 4; ++j) w[j] = (wp[j] && in) ? *(const bf16x8*)(wp[j] + k0) : zero;
+    for (int kk = 0; kk < BIG_K; kk += 32) {
+      bf16x8 a[4], w[4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+      for (int i = 0; i < 4; ++i) a[i] = *(const bf16x8*)(As + (wm * 64 + i * 16 + lr) * BIG_LD + kk + kq * 8);
 #pragma unroll
-      for (int j = 0; j < 4; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i], w[j], acc[i][j], 0, 0, 0);
+      for (int j = 0; j < 4; ++j) {
+        // gated: fragments 0, 1 are gate columns, 2, 3 the up columns of the same numbers
+        const int row = GATED ? (j >> 1) * 64 + wn * 32 + (j & 1) * 16 + lr : wn * 64 + j * 16 + lr;
+        w[j] = *(const bf16x8*)(Ws + row * BIG_LD + kk + kq * 8);
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i], w[j], acc[i][j], 0, 0, 0);
+    }
   }
   O* C = (O*)p.C + (experts ? 0 : (int64_t)tl.z * p.c_zs);
 #pragma unroll
