@@ -396,6 +396,195 @@ __global__ void __launch_bounds__(256) latent_attn_mfma_kernel(
   }
 }
 
+// Steps with prompt portions, keys and values shared through LDS: the four waves of a workgroup take four consecutive row
+// tiles of one request (64 rows) and walk the keys together; each block of 32 keys is brought into LDS once by the
+// whole workgroup (its rows, and its latents transposed, both in 16-byte pieces) and every wave takes its MFMA operands
+// from there, its queries too. The pieces of the next block are loaded into registers before a block is multiplied and
+// written to LDS after it, so a block's trip to memory is hidden behind the block before. A wave whose rows lie before a
+// block skips the arithmetic of that block, not the staging.
+template <int NT>
+__global__ void __launch_bounds__(256) latent_attn_lds_kernel(
+    const bf16* __restrict__ qa, int64_t ld_qa, bf16* __restrict__ out, int64_t ld_out, const bf16* __restrict__ cache,
+    const bf16* __restrict__ cache_t, const int32_t* __restrict__ block_table, int64_t max_blocks,
+    const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ seq_lens, int num_reqs, float scale_log2,
+    int window, int H, int R, int dr, int page, int page_shift) {
+  constexpr int NC = NT / 2 + 4;
+  constexpr int LDV = 40;              // a staged value row: 32 keys and 8 of padding
+  extern __shared__ __attribute__((aligned(16))) bf16 stage[];
+  const int DK = R + dr, LDK = DK + 8;
+  bf16* Ks = stage;                    // [32][LDK]
+  bf16* Vs = stage + 32 * LDK;         // [R][LDV]
+  // which request and which of its groups of four row tiles
+  int grp = blockIdx.x, b = -1, q_len = 0;
+  {
+    const int ln = threadIdx.x & 63;
+    for (int b0 = 0; b0 < num_reqs && b < 0; b0 += 64) {
+      const int mine = b0 + ln < num_reqs ? cu_seqlens[b0 + ln + 1] - cu_seqlens[b0 + ln] : 0;
+      int upto = (mine * H + 63) >> 6;
+#pragma unroll
+      for (int o = 1; o < 64; o <<= 1) {
+        const int v = __shfl_up(upto, o, 64);
+        if (ln >= o) upto += v;
+      }
+      const unsigned long long holds = __ballot(grp < upto);
+      if (holds) {
+        const int at = __ffsll((long long)holds) - 1;
+        b = b0 + at;
+        q_len = __shfl(mine, at, 64);
+        grp -= at ? __shfl(upto, at - 1, 64) : 0;
+      } else {
+        grp -= __shfl(upto, 63, 64);
+      }
+    }
+  }
+  if (b < 0) return;   // (the whole workgroup: every wave counts the same)
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, lr = lane & 15, g = lane >> 4;
+  const int start = seq_lens[b] - q_len;
+  const int all_rows = q_len * H;
+  const int row0 = (grp * 4 + wave) * 16;
+  const int nrows = all_rows - row0 < 16 ? all_rows - row0 : 16;   // <= 0: this wave has no rows, it only stages
+  const bool rv = lr < nrows;
+  const int tok = rv ? (row0 + lr) / H : 0, head = rv ? (row0 + lr) % H : 0;
+  const int p = rv ? start + tok : -1;
+  const int my_last = nrows > 0 ? start + (row0 + nrows - 1) / H : -1;
+  // of the whole workgroup
+  const int g_row0 = grp * 64;
+  const int g_rows = all_rows - g_row0 < 64 ? all_rows - g_row0 : 64;
+  const int p_first = start + g_row0 / H, p_last = start + (g_row0 + g_rows - 1) / H;
+  const int first = window > 0 ? (p_first - window + 1 > 0 ? p_first - window + 1 : 0) : 0;
+  const int lowest = window > 0 ? (p - window + 1 > 0 ? p - window + 1 : 0) : 0;
+  const int kb0 = first & ~31;
+  const int nblk = (p_last - kb0) / 32 + 1;
+  const int32_t* bt = block_table + (int64_t)b * max_blocks;
+
+  bf16x8 zero;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) zero[i] = (bf16)0.f;
+  const int kp = DK >> 3;                      // 16-byte pieces of a key row
+  // this wave's queries wait in LDS (in registers they would leave no room for the next block's pieces)
+  bf16* Qs = stage + 32 * LDK + R * LDV + wave * 16 * LDK;    // [16][LDK]
+  for (int q = lane; q < 16 * kp; q += 64) {
+    const int row = q / kp, pc = q - row * kp;
+    bf16x8 v = zero;
+    if (row < nrows) {
+      const int r = row0 + row;
+      v = *(const bf16x8*)(qa + (int64_t)(cu_seqlens[b] + r / H) * ld_qa + (int64_t)(r % H) * DK + pc * 8);
+    }
+    *(bf16x8*)(Qs + row * LDK + pc * 8) = v;
+  }
+  f32x4 o[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t) o[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, l = 0.f;
+  const int kofs = 8 * (lr >> 2) + (lr & 3);   // row of a key tile -> key, as in the kernel above
+  const int lo8 = first & ~7, hi8 = p_last & ~7;
+  // a thread's pieces of a block: of its rows (piece q is row q / kp, piece q % kp) and of its latents transposed
+  // (piece q is latent entry q / 4, keys 8 (q % 4) .. + 7)
+  constexpr int KP = (32 * (2 * NT + 16) + 255) / 256, VP = (64 * NT + 255) / 256;
+  bf16x8 kn[KP], vn[VP];
+  // piece q of the rows is row q / kp: the division is the high half of a multiplication by ceil(2^32 / kp), worked out
+  // once (exact for the q < 32 kp and 2 <= kp < 300 that occur: R + dr is at least 16 and at most 640 here)
+  const unsigned recip = (unsigned)((0x100000000ull + (unsigned)kp - 1u) / (unsigned)kp);
+  const int pmask = page - 1;     // the page size is a power of two here
+  auto fetch = [&](int kb) {
+#pragma unroll
+    for (int u = 0; u < KP; ++u) {
+      const int q = u * 256 + (int)threadIdx.x;
+      if (q < 32 * kp) {
+        const int row = (int)__umulhi((unsigned)q, recip), col = (q - row * kp) * 8;
+        int key = kb + row;
+        key = key < first ? first : (key > p_last ? p_last : key);
+        kn[u] = *(const bf16x8*)(cache + ((int64_t)bt[key >> page_shift] * page + (key & pmask)) * DK + col);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < VP; ++u) {
+      const int q = u * 256 + (int)threadIdx.x;
+      if (q < 4 * R) {
+        int key = kb + 8 * (q & 3);
+        key = key < lo8 ? lo8 : (key > hi8 ? hi8 : key);
+        vn[u] = *(const bf16x8*)(cache_t + (((int64_t)bt[key >> page_shift] * R + (q >> 2)) << page_shift) + (key & pmask));
+      }
+    }
+  };
+  fetch(kb0);
+  for (int blk = 0; blk < nblk; ++blk) {
+    const int kb = kb0 + blk * 32;
+    __syncthreads();   // the block before has been read
+#pragma unroll
+    for (int u = 0; u < KP; ++u) {
+      const int q = u * 256 + (int)threadIdx.x;
+      if (q < 32 * kp) {
+        const int row = (int)__umulhi((unsigned)q, recip);
+        *(bf16x8*)(Ks + row * LDK + (q - row * kp) * 8) = kn[u];
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < VP; ++u) {
+      const int q = u * 256 + (int)threadIdx.x;
+      if (q < 4 * R) *(bf16x8*)(Vs + (q >> 2) * LDV + 8 * (q & 3)) = vn[u];
+    }
+    __syncthreads();
+    if (blk + 1 < nblk) fetch(kb + 32);    // the next block's pieces travel while this one is multiplied
+    if (kb > my_last) continue;    // (the wave: all its rows lie before this block; it still meets the barriers above)
+    f32x4 s[2] = {f32x4{0.f, 0.f, 0.f, 0.f}, f32x4{0.f, 0.f, 0.f, 0.f}};
+#pragma unroll
+    for (int c = 0; c < NC; ++c) {
+      if (32 * c < DK) {
+        const int d = 32 * c + 8 * g;
+        const int dc = d < DK ? d : 0;     // entries beyond the row: the query's count as zeros
+        bf16x8 qv = *(const bf16x8*)(Qs + lr * LDK + dc);
+        if (d >= DK) qv = zero;
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+          s[t] = mfma16(*(const bf16x8*)(Ks + (kofs + 4 * t) * LDK + dc), qv, s[t]);
+      }
+    }
+    float mx = -INFINITY;
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int key = kb + 8 * g + 4 * t + i;
+        const float v = (key <= p && key >= lowest) ? s[t][i] * scale_log2 : -INFINITY;
+        s[t][i] = v;
+        mx = fmaxf(mx, v);
+      }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float m_new = fmaxf(m, mx);
+    const float alpha = m == -INFINITY ? 0.f : exp2_of(m - m_new);
+    bf16x8 pb;
+    float psum = 0.f;
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float pv = s[t][i] == -INFINITY ? 0.f : exp2_of(s[t][i] - m_new);
+        psum += pv;
+        pb[4 * t + i] = (bf16)pv;
+      }
+    l = l * alpha + psum;
+    m = m_new;
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+      if (16 * t < R) o[t] = mfma16(*(const bf16x8*)(Vs + (16 * t + lr) * LDV + 8 * g), pb, o[t] * alpha);
+  }
+  l += __shfl_xor(l, 16, 64);
+  l += __shfl_xor(l, 32, 64);
+  if (!rv) return;
+  const float inv = l > 0.f ? 1.f / l : 0.f;
+  bf16* orow = out + (int64_t)(cu_seqlens[b] + tok) * ld_out + (int64_t)head * R;
+#pragma unroll
+  for (int t = 0; t < NT; ++t)
+    if (16 * t < R) {
+      bf16x4 y;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) y[i] = (bf16)(o[t][i] * inv);
+      *(bf16x4*)(orow + 16 * t + 4 * g) = y;
+    }
+}
+
 // One workgroup per (token, head) row: the parts' (max, sum, output) become the row's output. A part is R + 4 floats
 // (output, max, sum, two unused), so its rows are read 16 bytes a lane.
 __global__ void __launch_bounds__(128) latent_attn_merge_kernel(const float* __restrict__ part, bf16* __restrict__ out,
@@ -500,6 +689,32 @@ extern "C" int dinfer_latent_attn_mfma(const void* qa, int64_t ld_qa, void* out,
   const int64_t tiles = (tokens * heads + 15) / 16 + num_reqs;
   if (tiles > 0x7fffffff || splits > 65535) return ERR_UNSUPPORTED;
   const bool solo = tokens != num_reqs;      // some request brings more than one row
+  if (solo && (page_size & (page_size - 1)) == 0) {
+    const int page_shift = __builtin_ctz(page_size);
+    const int64_t groups = (tokens * heads + 63) / 64 + num_reqs;
+    if (groups > 0x7fffffff) return ERR_UNSUPPORTED;
+    const size_t bytes = ((size_t)(32 + 64) * (R + dr + 8) + (size_t)R * 40) * sizeof(bf16);   // keys, 4 x 16 queries, values
+    const float sl2 = scale * LOG2E;
+#define LDS_LAUNCH(NT)                                                                                                 \
+  do {                                                                                                                 \
+    static bool sized = false;                                                                                         \
+    if (!sized) {                                                                                                      \
+      if (hipFuncSetAttribute((const void*)latent_attn_lds_kernel<NT>, hipFuncAttributeMaxDynamicSharedMemorySize,     \
+                              160 * 1024 - 1024) != hipSuccess)                                                        \
+        return ERR_LAUNCH;                                                                                             \
+      sized = true;                                                                                                    \
+    }                                                                                                                  \
+    latent_attn_lds_kernel<NT><<<(unsigned)groups, 256, bytes, stream>>>(                                              \
+        (const bf16*)qa, ld_qa, (bf16*)out, ld_out, (const bf16*)cache, (const bf16*)cache_t, block_table, max_blocks, \
+        cu_seqlens, seq_lens, num_reqs, sl2, window, heads, R, dr, page_size, page_shift);                                      \
+  } while (0)
+    if (R <= 64) LDS_LAUNCH(4);
+    else if (R <= 128) LDS_LAUNCH(8);
+    else if (R <= 256) LDS_LAUNCH(16);
+    else LDS_LAUNCH(32);
+#undef LDS_LAUNCH
+    return launch_status();
+  }
   const dim3 grid((unsigned)(solo ? (tiles + 3) / 4 : tiles), (unsigned)(solo ? 1 : splits));
   const size_t lds = solo ? 0 : (size_t)16 * (R + 4) * sizeof(float);
   const float sl = scale * LOG2E;
