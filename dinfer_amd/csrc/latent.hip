@@ -552,23 +552,32 @@ __global__ void __launch_bounds__(256) latent_attn_lds_kernel(
       }
     mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
     mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-    const float m_new = fmaxf(m, mx);
-    const float alpha = m == -INFINITY ? 0.f : exp2_of(m - m_new);
+    // The running maximum follows the scores only when one of the wave's rows has outgrown it by more than 2^8 (or has
+    // none yet): the weights may then exceed 1, up to 256, which float sums and bf16 weights hold without loss, and
+    // the 4 x NT multiplications that bring the output to a new maximum are done on few blocks instead of on all.
+    if (__any(mx > m + 8.f)) {
+      const float m_new = fmaxf(m, mx);
+      const float alpha = m == -INFINITY ? 0.f : exp2_of(m - m_new);
+      l *= alpha;
+      m = m_new;
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+        if (16 * t < R) o[t] = o[t] * alpha;
+    }
     bf16x8 pb;
     float psum = 0.f;
 #pragma unroll
     for (int t = 0; t < 2; ++t)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const float pv = s[t][i] == -INFINITY ? 0.f : exp2_of(s[t][i] - m_new);
+        const float pv = s[t][i] == -INFINITY ? 0.f : exp2_of(s[t][i] - m);
         psum += pv;
         pb[4 * t + i] = (bf16)pv;
       }
-    l = l * alpha + psum;
-    m = m_new;
+    l += psum;
 #pragma unroll
     for (int t = 0; t < NT; ++t)
-      if (16 * t < R) o[t] = mfma16(*(const bf16x8*)(Vs + (16 * t + lr) * LDV + 8 * g), pb, o[t] * alpha);
+      if (16 * t < R) o[t] = mfma16(*(const bf16x8*)(Vs + (16 * t + lr) * LDV + 8 * g), pb, o[t]);
   }
   l += __shfl_xor(l, 16, 64);
   l += __shfl_xor(l, 32, 64);
