@@ -698,18 +698,21 @@ extern "C" int dinfer_latent_attn_mfma(const void* qa, int64_t ld_qa, void* out,
   const int64_t tiles = (tokens * heads + 15) / 16 + num_reqs;
   if (tiles > 0x7fffffff || splits > 65535) return ERR_UNSUPPORTED;
   const bool solo = tokens != num_reqs;      // some request brings more than one row
-  if (solo && (page_size & (page_size - 1)) == 0) {
+  // keys, 4 x 16 queries and values of a block in LDS: where that fits (and pages are a power of two) prompt portions
+  // take the kernel that shares them; else every wave walks its own keys
+  const size_t bytes = ((size_t)(32 + 64) * (R + dr + 8) + (size_t)R * 40) * sizeof(bf16);
+  constexpr size_t LDS_MOST = 160 * 1024 - 1024;
+  if (solo && (page_size & (page_size - 1)) == 0 && bytes <= LDS_MOST) {
     const int page_shift = __builtin_ctz(page_size);
     const int64_t groups = (tokens * heads + 63) / 64 + num_reqs;
     if (groups > 0x7fffffff) return ERR_UNSUPPORTED;
-    const size_t bytes = ((size_t)(32 + 64) * (R + dr + 8) + (size_t)R * 40) * sizeof(bf16);   // keys, 4 x 16 queries, values
     const float sl2 = scale * LOG2E;
 #define LDS_LAUNCH(NT)                                                                                                 \
   do {                                                                                                                 \
     static bool sized = false;                                                                                         \
     if (!sized) {                                                                                                      \
       if (hipFuncSetAttribute((const void*)latent_attn_lds_kernel<NT>, hipFuncAttributeMaxDynamicSharedMemorySize,     \
-                              160 * 1024 - 1024) != hipSuccess)                                                        \
+                              (int)LDS_MOST) != hipSuccess)                                                             \
         return ERR_LAUNCH;                                                                                             \
       sized = true;                                                                                                    \
     }                                                                                                                  \

@@ -467,6 +467,8 @@ LATENT_CASES = [
     ([500, 64, 33], [37, 1, 33], 16, 128, 32, 8, 0, (0, 36, 9, 0)), # a portion behind a history, a single row, a prompt
     ([200, 90], [64, 2], 3, 48, 8, 8, 50, (0, 10, 1, 200 - 64 + 10 - 49)),   # a window: the oldest key a row still sees
     ([200, 90], [64, 2], 3, 48, 8, 8, 50, (0, 10, 1, 200 - 64 + 10 - 50)),   # ... and the first it does not
+    ([150, 70], [150, 3], 2, 512, 128, 16, 0, (0, 149, 1, 5)),     # the widest rows the matrix-core kernels take (no room in LDS)
+    ([260], [100], 5, 80, 24, 24, 0, (0, 99, 4, 160)),             # pages that are no power of two
 ]
 
 
