@@ -402,7 +402,8 @@ __global__ void __launch_bounds__(256) latent_attn_mfma_kernel(
 // from there, its queries too. The pieces of the next block are loaded into registers before a block is multiplied and
 // written to LDS after it, so a block's trip to memory is hidden behind the block before. A wave whose rows lie before a
 // block skips the arithmetic of that block, not the staging.
-template <int NT>
+// FULL: R + dr is a multiple of 32, so no chunk of a row is cut short (no selects, LDS offsets known at compile time).
+template <int NT, bool FULL>
 __global__ void __launch_bounds__(256) latent_attn_lds_kernel(
     const bf16* __restrict__ qa, int64_t ld_qa, bf16* __restrict__ out, int64_t ld_out, const bf16* __restrict__ cache,
     const bf16* __restrict__ cache_t, const int32_t* __restrict__ block_table, int64_t max_blocks,
@@ -414,8 +415,9 @@ __global__ void __launch_bounds__(256) latent_attn_lds_kernel(
   const int DK = R + dr, LDK = DK + 8;
   bf16* Ks = stage;                    // [32][LDK]
   bf16* Vs = stage + 32 * LDK;         // [R][LDV]
-  // which request and which of its groups of four row tiles
-  int grp = blockIdx.x, b = -1, q_len = 0;
+  // which request and which of its groups of four row tiles; the last groups of a prompt walk the most keys and start
+  // first, so that the short ones fill the gaps at the end
+  int grp = (int)gridDim.x - 1 - (int)blockIdx.x, b = -1, q_len = 0;
   {
     const int ln = threadIdx.x & 63;
     for (int b0 = 0; b0 < num_reqs && b < 0; b0 += 64) {
@@ -447,6 +449,7 @@ __global__ void __launch_bounds__(256) latent_attn_lds_kernel(
   const int tok = rv ? (row0 + lr) / H : 0, head = rv ? (row0 + lr) % H : 0;
   const int p = rv ? start + tok : -1;
   const int my_last = nrows > 0 ? start + (row0 + nrows - 1) / H : -1;
+  const int w_pmin = start + row0 / H;     // the earliest position among the wave's rows
   // of the whole workgroup
   const int g_row0 = grp * 64;
   const int g_rows = all_rows - g_row0 < 64 ? all_rows - g_row0 : 64;
@@ -486,24 +489,37 @@ __global__ void __launch_bounds__(256) latent_attn_lds_kernel(
   // once (exact for the q < 32 kp and 2 <= kp < 300 that occur: R + dr is at least 16 and at most 640 here)
   const unsigned recip = (unsigned)((0x100000000ull + (unsigned)kp - 1u) / (unsigned)kp);
   const int pmask = page - 1;     // the page size is a power of two here
+  const int page_lo = first >> page_shift, page_hi = p_last >> page_shift;
   auto fetch = [&](int kb) {
+    // the block's pages (up to four where pages are shorter than a block): the same for every lane, so their table
+    // entries and base offsets are scalar work; a page beyond the request's keys is replaced by its last one, whose
+    // rows exist (what they hold is masked)
+    int64_t pid[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      int pg = ((kb + (j << page_shift)) >> page_shift);
+      pg = pg < page_lo ? page_lo : (pg > page_hi ? page_hi : pg);
+      pid[j] = __builtin_amdgcn_readfirstlane(bt[pg]);
+    }
+    const int kbm = kb & pmask;
 #pragma unroll
     for (int u = 0; u < KP; ++u) {
       const int q = u * 256 + (int)threadIdx.x;
       if (q < 32 * kp) {
         const int row = (int)__umulhi((unsigned)q, recip), col = (q - row * kp) * 8;
-        int key = kb + row;
-        key = key < first ? first : (key > p_last ? p_last : key);
-        kn[u] = *(const bf16x8*)(cache + ((int64_t)bt[key >> page_shift] * page + (key & pmask)) * DK + col);
+        const int j = (kbm + row) >> page_shift;      // 0 .. 3 (0 where a page holds the whole block)
+        const int64_t pg = j == 0 ? pid[0] : j == 1 ? pid[1] : j == 2 ? pid[2] : pid[3];
+        kn[u] = *(const bf16x8*)(cache + ((pg << page_shift) + ((kbm + row) & pmask)) * DK + col);
       }
     }
 #pragma unroll
     for (int u = 0; u < VP; ++u) {
       const int q = u * 256 + (int)threadIdx.x;
       if (q < 4 * R) {
-        int key = kb + 8 * (q & 3);
-        key = key < lo8 ? lo8 : (key > hi8 ? hi8 : key);
-        vn[u] = *(const bf16x8*)(cache_t + (((int64_t)bt[key >> page_shift] * R + (q >> 2)) << page_shift) + (key & pmask));
+        const int k8 = kbm + 8 * (q & 3);
+        const int j = k8 >> page_shift;
+        const int64_t pg = j == 0 ? pid[0] : j == 1 ? pid[1] : j == 2 ? pid[2] : pid[3];
+        vn[u] = *(const bf16x8*)(cache_t + ((pg * R + (q >> 2)) << page_shift) + (k8 & pmask));
       }
     }
   };
@@ -531,25 +547,44 @@ __global__ void __launch_bounds__(256) latent_attn_lds_kernel(
 #pragma unroll
     for (int c = 0; c < NC; ++c) {
       if (32 * c < DK) {
-        const int d = 32 * c + 8 * g;
-        const int dc = d < DK ? d : 0;     // entries beyond the row: the query's count as zeros
-        bf16x8 qv = *(const bf16x8*)(Qs + lr * LDK + dc);
-        if (d >= DK) qv = zero;
+        if constexpr (FULL) {
+          const bf16x8 qv = *(const bf16x8*)(Qs + lr * LDK + 8 * g + 32 * c);
 #pragma unroll
-        for (int t = 0; t < 2; ++t)
-          s[t] = mfma16(*(const bf16x8*)(Ks + (kofs + 4 * t) * LDK + dc), qv, s[t]);
+          for (int t = 0; t < 2; ++t)
+            s[t] = mfma16(*(const bf16x8*)(Ks + (kofs + 4 * t) * LDK + 8 * g + 32 * c), qv, s[t]);
+        } else {
+          const int d = 32 * c + 8 * g;
+          const int dc = d < DK ? d : 0;     // entries beyond the row: the query's count as zeros
+          bf16x8 qv = *(const bf16x8*)(Qs + lr * LDK + dc);
+          if (d >= DK) qv = zero;
+#pragma unroll
+          for (int t = 0; t < 2; ++t)
+            s[t] = mfma16(*(const bf16x8*)(Ks + (kofs + 4 * t) * LDK + dc), qv, s[t]);
+        }
       }
     }
     float mx = -INFINITY;
+    // a block that every row of the wave sees whole needs no mask (most blocks of a long prompt)
+    const bool whole = nrows == 16 && kb + 31 <= w_pmin && (window == 0 || kb >= my_last - window + 1);
+    if (whole) {
 #pragma unroll
-    for (int t = 0; t < 2; ++t)
+      for (int t = 0; t < 2; ++t)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int key = kb + 8 * g + 4 * t + i;
-        const float v = (key <= p && key >= lowest) ? s[t][i] * scale_log2 : -INFINITY;
-        s[t][i] = v;
-        mx = fmaxf(mx, v);
-      }
+        for (int i = 0; i < 4; ++i) {
+          s[t][i] *= scale_log2;
+          mx = fmaxf(mx, s[t][i]);
+        }
+    } else {
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int key = kb + 8 * g + 4 * t + i;
+          const float v = (key <= p && key >= lowest) ? s[t][i] * scale_log2 : -INFINITY;
+          s[t][i] = v;
+          mx = fmaxf(mx, v);
+        }
+    }
     mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
     mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
     // The running maximum follows the scores only when one of the wave's rows has outgrown it by more than 2^8 (or has
@@ -707,24 +742,26 @@ extern "C" int dinfer_latent_attn_mfma(const void* qa, int64_t ld_qa, void* out,
     const int64_t groups = (tokens * heads + 63) / 64 + num_reqs;
     if (groups > 0x7fffffff) return ERR_UNSUPPORTED;
     const float sl2 = scale * LOG2E;
-#define LDS_LAUNCH(NT)                                                                                                 \
+#define LDS_LAUNCH_(NT, FULL)                                                                                                 \
   do {                                                                                                                 \
     static bool sized = false;                                                                                         \
     if (!sized) {                                                                                                      \
-      if (hipFuncSetAttribute((const void*)latent_attn_lds_kernel<NT>, hipFuncAttributeMaxDynamicSharedMemorySize,     \
+      if (hipFuncSetAttribute((const void*)latent_attn_lds_kernel<NT, FULL>, hipFuncAttributeMaxDynamicSharedMemorySize, \
                               (int)LDS_MOST) != hipSuccess)                                                             \
         return ERR_LAUNCH;                                                                                             \
       sized = true;                                                                                                    \
     }                                                                                                                  \
-    latent_attn_lds_kernel<NT><<<(unsigned)groups, 256, bytes, stream>>>(                                              \
+    latent_attn_lds_kernel<NT, FULL><<<(unsigned)groups, 256, bytes, stream>>>(                                        \
         (const bf16*)qa, ld_qa, (bf16*)out, ld_out, (const bf16*)cache, (const bf16*)cache_t, block_table, max_blocks, \
         cu_seqlens, seq_lens, num_reqs, sl2, window, heads, R, dr, page_size, page_shift);                                      \
   } while (0)
+#define LDS_LAUNCH(NT) do { if ((R + dr) % 32 == 0) LDS_LAUNCH_(NT, true); else LDS_LAUNCH_(NT, false); } while (0)
     if (R <= 64) LDS_LAUNCH(4);
     else if (R <= 128) LDS_LAUNCH(8);
     else if (R <= 256) LDS_LAUNCH(16);
     else LDS_LAUNCH(32);
 #undef LDS_LAUNCH
+#undef LDS_LAUNCH_
     return launch_status();
   }
   const dim3 grid((unsigned)(solo ? (tiles + 3) / 4 : tiles), (unsigned)(solo ? 1 : splits));
