@@ -358,6 +358,23 @@ def test_greedy_generation_through_the_engine(models, name):
             ids.append(tok)
 
 
+@pytest.mark.parametrize("name", ["K1", "K3"])
+def test_bfloat16_generation_is_the_same_from_graphs(models, name):
+    """Greedy generation in bfloat16 through the engine, steps replayed from graphs (single rows and prompt portions whose
+    counts come up again) against the same engine launching every step eagerly: the same tokens, and graphs were used."""
+    from dinfer_amd import Engine, SamplingParams
+    d, cfg, _, page = models[name]
+    prompts = [tokens_for(cfg, 40, s) for s in range(1, 11)] + [tokens_for(cfg, n, 20 + n) for n in (9, 3)]
+    outs = []
+    for graphs in (True, False):
+        eng = Engine(str(d), dtype="bfloat16", max_model_len=128, max_num_seqs=2, block_size=page, num_blocks=64,
+                     max_num_batched_tokens=16, hip_graph=graphs, gemm_tuning="heuristic")
+        outs.append(eng.generate(prompts, SamplingParams(max_tokens=10, temperature=0.0)))
+        if graphs:
+            assert eng.runner._graphs and eng.runner.portion_replays > 0
+    assert outs[0] == outs[1]
+
+
 def test_config_round_trip_and_refusals(models):
     from dinfer_amd.config import ConfigError, load_config
     d, cfg, _, _ = models["K1"]
