@@ -38,10 +38,12 @@ _I32, _I64 = ctypes.c_int32, ctypes.c_int64
 
 @dataclass(frozen=True)
 class GroupSpec:
-    """window None: every key of the request is kept. window W: the last W keys."""
+    """window None: every key of the request is kept. window W: the last W keys, and the first keep_first keys
+    besides (their pages are never given back while the request lives)."""
     page_size: int
     num_blocks: int
     window: int | None = None
+    keep_first: int = 0
 
 
 class _PoolView:
@@ -75,6 +77,9 @@ class CacheManager:
                                  arr([g.num_blocks for g in self.groups]),
                                  arr([-1 if g.window is None else g.window for g in self.groups]), int(max_seqs),
                                  int(self.prefix_caching))
+        for g, spec in enumerate(self.groups):
+            if spec.keep_first:
+                native.checked("dh_cache_set_keep_first", self._h, g, int(spec.keep_first))
         self.max_seqs = max_seqs
         self.pools = [_PoolView(self, g) for g in range(n)]
         self._handles: dict = {}          # request id -> the number the core knows it by

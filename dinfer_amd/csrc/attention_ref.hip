@@ -8,6 +8,15 @@
 //   keys j in [max(0, p - window + 1), p]  (window 0: all keys up to p);
 //   s_j = scale * <q, k_j>;  P = softmax(s);  o = sum_j P_j v_j   (all float)
 //
+// Options (dinfer_attn_paged_ext; each is off at its zero):
+//   keep_first F   the keys j < F stay visible after the window has passed them (they keep their positions);
+//   sinks          one float a query head: exp(sink_h) is added to the softmax's denominator once; it has no key, no
+//                  value and is not scaled;
+//   slope_exp E    s_j -= 2^(-E (h + 1) / H) * (p - j): a bias that grows with the distance, steeper for low heads;
+//   v_dim          the value size where it differs from the key size;
+//   values in the key pages (v_cache null): a layer whose values are its keys stores them once;
+//   out_scale      o is multiplied by it on store.
+//
 // K and V are read from the cache pages through the request's block table
 // (K page [Hkv][D / 8][page][8], V page [Hkv][D][page]); the step's own tokens were
 // written there before this kernel runs.
@@ -29,7 +38,8 @@ __global__ void __launch_bounds__(WAVES * 64) attn_paged_ref_kernel(
     const S* __restrict__ q, int64_t ld_q, S* __restrict__ out, int64_t ld_out, const S* __restrict__ k_cache,
     const S* __restrict__ v_cache, const int32_t* __restrict__ block_table, int64_t max_blocks,
     const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ seq_lens, int num_reqs, float scale,
-    int window, int H, int Hkv, int D, int page) {
+    int window, int H, int Hkv, int D, int page, int keep_first, const float* __restrict__ sinks, float slope_exp,
+    int Dv, float out_scale) {
   __shared__ float qs[WAVES][MAX_D];
   __shared__ float ps[WAVES][64];
   const int t = blockIdx.x;
@@ -49,6 +59,9 @@ __global__ void __launch_bounds__(WAVES * 64) attn_paged_ref_kernel(
   const int first_key = window > 0 ? (p - window + 1 > 0 ? p - window + 1 : 0) : 0;
   const int32_t* bt = block_table + (int64_t)b * max_blocks;
   const int hk = live ? h / (H / Hkv) : 0;
+  const float slope = slope_exp != 0.f ? exp2f(-slope_exp * (float)(h + 1) / (float)H) : 0.f;
+  // two runs of keys: the kept first ones that the window has passed, then the window itself
+  const int kept = keep_first < first_key ? keep_first : first_key;
 
   if (live) {
     const S* qr = q + (int64_t)t * ld_q + (int64_t)h * D;
@@ -62,19 +75,20 @@ __global__ void __launch_bounds__(WAVES * 64) attn_paged_ref_kernel(
   for (int c = 0; c < NC; ++c) o[c] = 0.f;
   float m = -INFINITY, l = 0.f;
 
-  for (int j0 = first_key; j0 <= p; j0 += 64) {
+  for (int run = kept > 0 ? 0 : 1; run < 2; ++run)
+  for (int j0 = run ? first_key : 0, last = run ? p : kept - 1; j0 <= last; j0 += 64) {
     const int j = j0 + lane;
     float s = -INFINITY;
-    if (live && j <= p) {
+    if (live && j <= last) {
       const int blk = bt[j / page];
       const S* kr = k_cache + ((int64_t)blk * Hkv + hk) * page * D;  // the head's page
       const int off = j % page;
       float acc = 0.f;
       for (int d = 0; d < D; ++d) acc += qs[wave][d] * to_f32(kr[k_page_offset(off, d, page)]);
-      s = acc * scale;
+      s = acc * scale - slope * (float)(p - j);
     }
     const float m_new = fmaxf(m, wave_max(s));
-    const float pj = (live && j <= p) ? expf(s - m_new) : 0.f;
+    const float pj = (live && j <= last) ? expf(s - m_new) : 0.f;
     const float alpha = expf(m - m_new);  // m = -inf on the first tile: alpha = 0
     l = l * alpha + wave_sum(pj);
     m = m_new;
@@ -82,16 +96,17 @@ __global__ void __launch_bounds__(WAVES * 64) attn_paged_ref_kernel(
     ps[wave][lane] = pj;
     __syncthreads();
     if (live) {
-      const int n = p - j0 + 1 < 64 ? p - j0 + 1 : 64;
+      const int n = last - j0 + 1 < 64 ? last - j0 + 1 : 64;
 #pragma unroll
       for (int c = 0; c < NC; ++c) {
         const int d = lane + 64 * c;
-        if (d < D) {
+        if (d < Dv) {
           float acc = o[c] * alpha;
           for (int jj = 0; jj < n; ++jj) {
             const int key = j0 + jj;
             const int blk = bt[key / page];
-            const S* vr = v_cache + (((int64_t)blk * Hkv + hk) * D + d) * page + (key % page);
+            const S* vr = v_cache ? v_cache + (((int64_t)blk * Hkv + hk) * Dv + d) * page + (key % page)
+                                  : k_cache + ((int64_t)blk * Hkv + hk) * page * D + k_page_offset(key % page, d, page);
             acc += ps[wave][jj] * to_f32(*vr);
           }
           o[c] = acc;
@@ -99,13 +114,21 @@ __global__ void __launch_bounds__(WAVES * 64) attn_paged_ref_kernel(
       }
     }
   }
+  if (live && sinks) {  // the sink joins the denominator as one more term
+    const float sk = sinks[h];
+    const float m_new = fmaxf(m, sk);
+    const float alpha = expf(m - m_new);
+    l = l * alpha + expf(sk - m_new);
+#pragma unroll
+    for (int c = 0; c < NC; ++c) o[c] *= alpha;
+  }
   if (live) {
-    S* orow = out + (int64_t)t * ld_out + (int64_t)h * D;
-    const float inv = l > 0.f ? 1.f / l : 0.f;
+    S* orow = out + (int64_t)t * ld_out + (int64_t)h * Dv;
+    const float inv = l > 0.f ? out_scale / l : 0.f;
 #pragma unroll
     for (int c = 0; c < NC; ++c) {
       const int d = lane + 64 * c;
-      if (d < D) orow[d] = from_f32<S>(o[c] * inv);
+      if (d < Dv) orow[d] = from_f32<S>(o[c] * inv);
     }
   }
 }
@@ -129,7 +152,30 @@ extern "C" int dinfer_attn_paged_ref(int dtype, const void* q, int64_t ld_q, voi
   DINFER_DISPATCH_DTYPE(dtype, {
     attn_paged_ref_kernel<S><<<grid, WAVES * 64, 0, stream>>>(
         (const S*)q, ld_q, (S*)out, ld_out, (const S*)k_cache, (const S*)v_cache, block_table, max_blocks, cu_seqlens,
-        seq_lens, num_reqs, scale, window, heads, kv_heads, head_dim, page_size);
+        seq_lens, num_reqs, scale, window, heads, kv_heads, head_dim, page_size, 0, nullptr, 0.f, head_dim, 1.f);
+  });
+  return launch_status();
+}
+
+// The same with the options of the header. out [T, ld_out] holds head h at column h * v_dim. v_cache null: the values
+// are the keys and are read from the key pages (v_dim must equal head_dim).
+extern "C" int dinfer_attn_paged_ext(int dtype, const void* q, int64_t ld_q, void* out, int64_t ld_out,
+                                     const void* k_cache, const void* v_cache, const int32_t* block_table,
+                                     int64_t max_blocks, const int32_t* cu_seqlens, const int32_t* seq_lens,
+                                     int num_reqs, int64_t tokens, float scale, int window, int keep_first,
+                                     const float* sinks, float slope_exp, int heads, int kv_heads, int head_dim,
+                                     int v_dim, int page_size, float out_scale, hipStream_t stream) {
+  if (tokens <= 0 || num_reqs <= 0) return OK;
+  if (heads <= 0 || kv_heads <= 0 || heads % kv_heads != 0 || head_dim <= 0 || v_dim <= 0 || page_size <= 0 ||
+      max_blocks <= 0 || window < 0 || keep_first < 0 || tokens > 0x7fffffff || (!v_cache && v_dim != head_dim))
+    return ERR_BAD_SHAPE;
+  if (head_dim > MAX_D || v_dim > MAX_D) return ERR_UNSUPPORTED;
+  const dim3 grid((unsigned)tokens, (unsigned)((heads + WAVES - 1) / WAVES));
+  DINFER_DISPATCH_DTYPE(dtype, {
+    attn_paged_ref_kernel<S><<<grid, WAVES * 64, 0, stream>>>(
+        (const S*)q, ld_q, (S*)out, ld_out, (const S*)k_cache, (const S*)v_cache, block_table, max_blocks, cu_seqlens,
+        seq_lens, num_reqs, scale, window, heads, kv_heads, head_dim, page_size, window > 0 ? keep_first : 0, sinks,
+        slope_exp, v_dim, out_scale);
   });
   return launch_status();
 }

@@ -35,6 +35,7 @@ SOURCES = {
     "gemm_wide": "gemm_wide.hip",
     "latent": "latent.hip",
     "grouped": "grouped.hip",
+    "delta": "delta.hip",
     "sampling": "sampling.hip",
     "ceilings": "ceilings.hip",
     "host": "host/api.cpp",

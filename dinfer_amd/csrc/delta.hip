@@ -1,0 +1,333 @@
+// Gated delta rule: a recurrent mixer whose state is one matrix S [D, V] a head and request, in float.
+//
+//   per token, per head:   S <- g S;   u = beta (v - S^T k);   S <- S + k u^T;   o = S^T q
+//
+// with q and k unit vectors (q times q_scale), g in (0, 1) a decay and beta in (0, 1) a step size, all float. q, k and
+// v come out of a short causal convolution over time (a few taps a channel) and silu; the convolution's last
+// taps - 1 inputs are state as well. Four kernels serve prompt portions and single decoded rows alike:
+//
+//   delta_prep         one wave a (token, head of q, k or v): convolution over the step's rows and the request's
+//                      stored inputs, silu, unit norm of q and k; one more wave a token makes beta and g. Float out.
+//   delta_recurrence   the recurrence, token by token, for one request, one head and 32 columns of S a workgroup.
+//                      A thread owns a strip of rows of one column: lanes 0..7 of a group of eight share a column
+//                      and meet by three shuffles for each of the two products with S. k, q, v, beta and g of 16
+//                      tokens wait in LDS while the next 16 are on their way in registers.
+//   delta_conv_update  moves the step's last taps - 1 inputs into the request's stored inputs (after prep has read
+//                      the old ones).
+//   delta_out          o / rms(o) * w * silu(gate) per head, one wave a (token, head), rounded once on store.
+//
+// S is stored transposed, [slot][head][V][D]: a thread's strip is contiguous, a wave reads and writes 2 KB to 8 KB in
+// one piece, which is what a decode step (one token a request: all of S in and out) is made of.
+// A request whose step starts at position 0 starts from S = 0 and zero stored inputs, whatever its slot held.
+// Nothing depends on how a request's tokens were cut into steps: every token does the same arithmetic in the same order.
+#include "common.cuh"
+
+using namespace dinfer;
+
+namespace {
+
+constexpr int WAVES = 4;
+constexpr int MAX_HEAD = 512;   // the largest D or V of the prep and out kernels (8 values a lane)
+constexpr int MAX_TAPS = 16;
+constexpr int CH = 16;          // tokens of a chunk in the recurrence
+constexpr int COLS = 32;        // columns of S a workgroup
+
+__device__ __forceinline__ int request_of(const int32_t* __restrict__ cu, int num_reqs, int t) {
+  int lo = 0, hi = num_reqs - 1;
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if (cu[mid] <= t) lo = mid; else hi = mid - 1;
+  }
+  return lo;
+}
+
+__device__ __forceinline__ float silu_f(float z) { return z / (1.f + expf(-z)); }
+__device__ __forceinline__ float sigmoid_f(float z) { return 1.f / (1.f + expf(-z)); }
+__device__ __forceinline__ float softplus_f(float z) { return z > 20.f ? z : log1pf(expf(z)); }
+
+// work [T, ldw] float: q (G D) | k (G D) | v (H V) | beta (H) | g (H)
+template <class S>
+__global__ void __launch_bounds__(WAVES * 64) delta_prep_kernel(
+    const S* __restrict__ proj, int64_t ld, int64_t qkv_off, int64_t b_off, int64_t a_off,
+    const float* __restrict__ taps, const float* __restrict__ a_log, const float* __restrict__ dt_bias,
+    const S* __restrict__ conv_state, const int32_t* __restrict__ slots, const int32_t* __restrict__ cu,
+    const int32_t* __restrict__ seq_lens, float* __restrict__ work, int64_t ldw, int num_reqs, int G, int H, int D,
+    int V, int K, float eps, float q_scale) {
+  const int t = blockIdx.x;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int item = blockIdx.y * WAVES + wave;
+  const int items = 2 * G + H + 1;
+  if (item >= items) return;
+  const int b = request_of(cu, num_reqs, t);
+  const int i = t - cu[b];                                   // index of the token in its request's rows of this step
+  const int start = seq_lens[b] - (cu[b + 1] - cu[b]);       // position of the request's first row of this step
+  const S* row = proj + (int64_t)t * ld;
+  float* wr = work + (int64_t)t * ldw;
+  const int gd = 2 * G * D;
+  if (item == items - 1) {                                   // the step size and the decay of every head
+    for (int h = lane; h < H; h += 64) {
+      wr[gd + H * V + h] = sigmoid_f(to_f32(row[b_off + h]));
+      const float sp = softplus_f(to_f32(row[a_off + h]) + dt_bias[h]);
+      wr[gd + H * V + H + h] = expf(-expf(a_log[h]) * sp);
+    }
+    return;
+  }
+  const bool qk = item < 2 * G;
+  const int c0 = qk ? item * D : gd + (item - 2 * G) * V;   // first channel of the head
+  const int n = qk ? D : V;
+  const S* old = (K > 1 && start > 0) ? conv_state + (int64_t)slots[b] * (gd + H * V) * (K - 1) : nullptr;
+  constexpr int PER = MAX_HEAD / 64;
+  float y[PER];
+  float ss = 0.f;
+#pragma unroll
+  for (int e = 0; e < PER; ++e) {
+    const int d = lane + 64 * e;
+    y[e] = 0.f;
+    if (d < n) {
+      const int c = c0 + d;
+      float acc = 0.f;
+      for (int j = K - 1; j >= 0; --j) {                     // the oldest input first
+        float x = 0.f;
+        if (i - j >= 0) x = to_f32(row[qkv_off + c - (int64_t)j * ld]);
+        else if (old) x = to_f32(old[(int64_t)c * (K - 1) + (K - 1 + i - j)]);
+        acc = __builtin_fmaf(taps[(int64_t)c * K + (K - 1 - j)], x, acc);
+      }
+      y[e] = silu_f(acc);
+      ss = __builtin_fmaf(y[e], y[e], ss);
+    }
+  }
+  float mul = 1.f;
+  if (qk) {
+    ss = wave_sum(ss);
+    mul = (item < G ? q_scale : 1.f) / sqrtf(ss + eps);
+  }
+#pragma unroll
+  for (int e = 0; e < PER; ++e) {
+    const int d = lane + 64 * e;
+    if (d < n) wr[c0 + d] = y[e] * mul;
+  }
+}
+
+template <class S>
+__global__ void __launch_bounds__(256) delta_conv_update_kernel(const S* __restrict__ proj, int64_t ld, int64_t qkv_off,
+                                                                S* __restrict__ conv_state,
+                                                                const int32_t* __restrict__ slots,
+                                                                const int32_t* __restrict__ cu,
+                                                                const int32_t* __restrict__ seq_lens, int C, int K) {
+  const int b = blockIdx.x;
+  const int c = blockIdx.y * 256 + threadIdx.x;
+  if (c >= C) return;
+  const int t0 = cu[b], n = cu[b + 1] - t0;
+  const int start = seq_lens[b] - n;
+  S* st = conv_state + ((int64_t)slots[b] * C + c) * (K - 1);
+  // entry s holds the input of row n - (K - 1) + s of this step; rows before the step come from the old entries,
+  // which lie further back than the entry being written (n >= 1), so ascending order reads before it overwrites
+  for (int s = 0; s < K - 1; ++s) {
+    const int i = n - (K - 1) + s;
+    S x;
+    if (i >= 0) x = proj[(int64_t)(t0 + i) * ld + qkv_off + c];
+    else x = start > 0 ? st[K - 1 + i] : from_f32<S>(0.f);
+    st[s] = x;
+  }
+}
+
+template <int RPT>
+__global__ void __launch_bounds__(256) delta_recurrence_kernel(
+    const float* __restrict__ work, int64_t ldw, float* __restrict__ state, const int32_t* __restrict__ slots,
+    const int32_t* __restrict__ cu, const int32_t* __restrict__ seq_lens, float* __restrict__ out, int64_t ld_out,
+    int G, int H, int D, int V) {
+  constexpr int DP = 8 * RPT;
+  __shared__ float ks[CH][DP];
+  __shared__ float qs[CH][DP];
+  __shared__ float vs[CH][COLS];
+  __shared__ float bs[CH], gs[CH];
+  const int b = blockIdx.x, h = blockIdx.y;
+  const int tid = threadIdx.x;
+  const int rg = tid & 7, cj = tid >> 3;
+  const int j = blockIdx.z * COLS + cj;
+  const int t0 = cu[b], n = cu[b + 1] - t0;
+  const int start = seq_lens[b] - n;
+  const int g = h / (H / G);
+  const int gd = 2 * G * D;
+  const bool col_ok = j < V;
+  float* sp = state + ((((int64_t)slots[b] * H + h) * V + (col_ok ? j : 0)) * D) + rg * RPT;
+  float S[RPT];
+#pragma unroll
+  for (int i = 0; i < RPT; ++i) S[i] = (start > 0 && col_ok && rg * RPT + i < D) ? sp[i] : 0.f;
+
+  // what a thread carries of the next chunk: RPT / 2 entries of k and of q, two of v, one of beta or g
+  constexpr int PK = (CH * DP) / 256;
+  float pk[PK], pq[PK], pv[2], pbg = 0.f;
+  const float* wk = work + (int64_t)t0 * ldw;
+  auto fetch = [&](int ct) {
+#pragma unroll
+    for (int e = 0; e < PK; ++e) {
+      const int idx = tid + e * 256;
+      const int tok = idx / DP, d = idx % DP;
+      const bool ok = ct + tok < n && d < D;
+      const float* r = wk + (int64_t)(ct + tok) * ldw + g * D + d;
+      pk[e] = ok ? r[G * D] : 0.f;
+      pq[e] = ok ? r[0] : 0.f;
+    }
+#pragma unroll
+    for (int e = 0; e < 2; ++e) {
+      const int idx = tid + e * 256;
+      const int tok = idx / COLS, c = idx % COLS;
+      const int col = blockIdx.z * COLS + c;
+      pv[e] = (ct + tok < n && col < V) ? wk[(int64_t)(ct + tok) * ldw + gd + h * V + col] : 0.f;
+    }
+    if (tid < 2 * CH) {
+      const int tok = tid % CH;
+      pbg = ct + tok < n ? wk[(int64_t)(ct + tok) * ldw + gd + H * V + (tid < CH ? 0 : H) + h] : 0.f;
+    }
+  };
+  fetch(0);
+  for (int ct = 0; ct < n; ct += CH) {
+    __syncthreads();  // the chunk before has been consumed
+#pragma unroll
+    for (int e = 0; e < PK; ++e) {
+      const int idx = tid + e * 256;
+      ks[idx / DP][idx % DP] = pk[e];
+      qs[idx / DP][idx % DP] = pq[e];
+    }
+#pragma unroll
+    for (int e = 0; e < 2; ++e) {
+      const int idx = tid + e * 256;
+      vs[idx / COLS][idx % COLS] = pv[e];
+    }
+    if (tid < CH) bs[tid] = pbg;
+    else if (tid < 2 * CH) gs[tid - CH] = pbg;
+    __syncthreads();
+    if (ct + CH < n) fetch(ct + CH);  // in flight while this chunk is worked through
+    const int m = n - ct < CH ? n - ct : CH;
+    for (int tok = 0; tok < m; ++tok) {
+      const float* kr = &ks[tok][rg * RPT];
+      const float* qr = &qs[tok][rg * RPT];
+      float dot = 0.f;
+#pragma unroll
+      for (int i = 0; i < RPT; ++i) dot = __builtin_fmaf(S[i], kr[i], dot);
+      dot += __shfl_xor(dot, 1, WAVE);
+      dot += __shfl_xor(dot, 2, WAVE);
+      dot += __shfl_xor(dot, 4, WAVE);
+      const float dec = gs[tok];
+      const float u = bs[tok] * (vs[tok][cj] - dec * dot);    // (g S)^T k = g (S^T k)
+      float o = 0.f;
+#pragma unroll
+      for (int i = 0; i < RPT; ++i) {
+        S[i] = __builtin_fmaf(kr[i], u, dec * S[i]);
+        o = __builtin_fmaf(S[i], qr[i], o);
+      }
+      o += __shfl_xor(o, 1, WAVE);
+      o += __shfl_xor(o, 2, WAVE);
+      o += __shfl_xor(o, 4, WAVE);
+      if (rg == 0 && col_ok) out[(int64_t)(t0 + ct + tok) * ld_out + h * V + j] = o;
+    }
+  }
+  if (col_ok) {
+#pragma unroll
+    for (int i = 0; i < RPT; ++i)
+      if (rg * RPT + i < D) sp[i] = S[i];
+  }
+}
+
+template <class S>
+__global__ void __launch_bounds__(WAVES * 64) delta_out_kernel(const float* __restrict__ o, int64_t ld_o,
+                                                               const S* __restrict__ proj, int64_t ld, int64_t g_off,
+                                                               const float* __restrict__ w, S* __restrict__ out,
+                                                               int64_t ld_out, int64_t col_off, int H, int V, float eps,
+                                                               float out_scale) {
+  const int t = blockIdx.x;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int h = blockIdx.y * WAVES + wave;
+  if (h >= H) return;
+  constexpr int PER = MAX_HEAD / 64;
+  float x[PER];
+  float ss = 0.f;
+#pragma unroll
+  for (int e = 0; e < PER; ++e) {
+    const int d = lane + 64 * e;
+    x[e] = d < V ? o[(int64_t)t * ld_o + h * V + d] : 0.f;
+    ss = __builtin_fmaf(x[e], x[e], ss);
+  }
+  const float inv = 1.f / sqrtf(wave_sum(ss) / (float)V + eps);
+#pragma unroll
+  for (int e = 0; e < PER; ++e) {
+    const int d = lane + 64 * e;
+    if (d < V) {
+      const float gate = silu_f(to_f32(proj[(int64_t)t * ld + g_off + h * V + d]));
+      out[(int64_t)t * ld_out + col_off + h * V + d] = from_f32<S>(x[e] * inv * w[d] * gate * out_scale);
+    }
+  }
+}
+
+}  // namespace
+
+// proj [T, ld]: the step's fused projection; q (G D) | k (G D) | v (H V) lie together from column qkv_off, the H
+// step-size logits at b_off, the H decay logits at a_off. taps [2 G D + H V, K] float, the last column the current
+// token's. a_log, dt_bias [H] float. conv_state [slots, 2 G D + H V, K - 1] in the step's dtype (unused with K = 1).
+// work [T, ldw] float, ldw >= 2 G D + H V + 2 H.
+extern "C" int dinfer_delta_prep(int dtype, const void* proj, int64_t ld, int64_t qkv_off, int64_t b_off, int64_t a_off,
+                                 const float* taps, const float* a_log, const float* dt_bias, const void* conv_state,
+                                 const int32_t* state_slots, const int32_t* cu_seqlens, const int32_t* seq_lens,
+                                 float* work, int64_t ldw, int num_reqs, int64_t tokens, int G, int H, int D, int V,
+                                 int K, float eps, float q_scale, hipStream_t stream) {
+  if (tokens <= 0 || num_reqs <= 0) return OK;
+  if (G <= 0 || H <= 0 || H % G || D <= 0 || V <= 0 || K <= 0 || tokens > 0x7fffffff ||
+      ldw < 2 * (int64_t)G * D + (int64_t)H * V + 2 * H)
+    return ERR_BAD_SHAPE;
+  if (D > MAX_HEAD || V > MAX_HEAD || K > MAX_TAPS) return ERR_UNSUPPORTED;
+  const dim3 grid((unsigned)tokens, (unsigned)((2 * G + H + 1 + WAVES - 1) / WAVES));
+  DINFER_DISPATCH_DTYPE(dtype, {
+    delta_prep_kernel<S><<<grid, WAVES * 64, 0, stream>>>((const S*)proj, ld, qkv_off, b_off, a_off, taps, a_log,
+                                                          dt_bias, (const S*)conv_state, state_slots, cu_seqlens,
+                                                          seq_lens, work, ldw, num_reqs, G, H, D, V, K, eps, q_scale);
+  });
+  return launch_status();
+}
+
+extern "C" int dinfer_delta_conv_update(int dtype, const void* proj, int64_t ld, int64_t qkv_off, void* conv_state,
+                                        const int32_t* state_slots, const int32_t* cu_seqlens, const int32_t* seq_lens,
+                                        int num_reqs, int channels, int K, hipStream_t stream) {
+  if (num_reqs <= 0 || K <= 1) return OK;
+  if (channels <= 0 || K > MAX_TAPS) return ERR_BAD_SHAPE;
+  const dim3 grid((unsigned)num_reqs, (unsigned)((channels + 255) / 256));
+  DINFER_DISPATCH_DTYPE(dtype, {
+    delta_conv_update_kernel<S><<<grid, 256, 0, stream>>>((const S*)proj, ld, qkv_off, (S*)conv_state, state_slots,
+                                                          cu_seqlens, seq_lens, channels, K);
+  });
+  return launch_status();
+}
+
+// state [slots, H, V, D] float (S transposed); out [T, ld_out] float, head h at column h V.
+extern "C" int dinfer_delta_recurrence(const float* work, int64_t ldw, float* state, const int32_t* state_slots,
+                                       const int32_t* cu_seqlens, const int32_t* seq_lens, float* out, int64_t ld_out,
+                                       int num_reqs, int G, int H, int D, int V, hipStream_t stream) {
+  if (num_reqs <= 0) return OK;
+  if (G <= 0 || H <= 0 || H % G || D <= 0 || V <= 0 || num_reqs > 0x7fffffff || H > 65535) return ERR_BAD_SHAPE;
+  if (D > 256) return ERR_UNSUPPORTED;
+  const dim3 grid((unsigned)num_reqs, (unsigned)H, (unsigned)((V + COLS - 1) / COLS));
+#define DELTA_REC(R_)                                                                                               \
+  delta_recurrence_kernel<R_><<<grid, 256, 0, stream>>>(work, ldw, state, state_slots, cu_seqlens, seq_lens, out, \
+                                                        ld_out, G, H, D, V)
+  if (D <= 32) DELTA_REC(4);
+  else if (D <= 64) DELTA_REC(8);
+  else if (D <= 128) DELTA_REC(16);
+  else DELTA_REC(32);
+#undef DELTA_REC
+  return launch_status();
+}
+
+// out[t, col_off + h V + d] = o[t, h V + d] / sqrt(mean_d o^2 + eps) * w[d] * silu(proj[t, g_off + h V + d]) * out_scale
+extern "C" int dinfer_delta_out(int dtype, const float* o, int64_t ld_o, const void* proj, int64_t ld, int64_t g_off,
+                                const float* w, void* out, int64_t ld_out, int64_t col_off, int64_t tokens, int H, int V,
+                                float eps, float out_scale, hipStream_t stream) {
+  if (tokens <= 0) return OK;
+  if (H <= 0 || V <= 0 || tokens > 0x7fffffff) return ERR_BAD_SHAPE;
+  if (V > MAX_HEAD) return ERR_UNSUPPORTED;
+  const dim3 grid((unsigned)tokens, (unsigned)((H + WAVES - 1) / WAVES));
+  DINFER_DISPATCH_DTYPE(dtype, {
+    delta_out_kernel<S><<<grid, WAVES * 64, 0, stream>>>(o, ld_o, (const S*)proj, ld, g_off, w, (S*)out, ld_out,
+                                                         col_off, H, V, eps, out_scale);
+  });
+  return launch_status();
+}

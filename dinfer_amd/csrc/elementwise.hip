@@ -246,3 +246,65 @@ extern "C" int dinfer_act(int dtype, int act, const void* in, int64_t ld_in, voi
   }
   return launch_status();
 }
+
+namespace {
+
+template <class S>
+__global__ void __launch_bounds__(256) axpby_kernel(const S* __restrict__ a, int64_t ld_a, float alpha,
+                                                    const S* __restrict__ b, int64_t ld_b, float beta,
+                                                    S* __restrict__ out, int64_t ld_out, int64_t cols) {
+  const int64_t t = blockIdx.y;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < cols; i += (int64_t)gridDim.x * blockDim.x)
+    out[t * ld_out + i] = from_f32<S>(alpha * to_f32(a[t * ld_a + i]) + beta * to_f32(b[t * ld_b + i]));
+}
+
+template <class SX, class SA, class SV>
+__global__ void __launch_bounds__(256) add_rows_kernel(SX* __restrict__ x, int64_t ld_x, const SA* __restrict__ a,
+                                                       int64_t ld_a, const SV* __restrict__ vec, int64_t width) {
+  const int64_t t = blockIdx.y;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < width; i += (int64_t)gridDim.x * blockDim.x) {
+    float v = to_f32(x[t * ld_x + i]);
+    if (a) v += to_f32(a[t * ld_a + i]);      // in this order: the rows first, then the vector
+    if (vec) v += to_f32(vec[i]);
+    x[t * ld_x + i] = from_f32<SX>(v);
+  }
+}
+
+}  // namespace
+
+// out[t, i] = alpha a[t, i] + beta b[t, i] (float arithmetic, one rounding); out may be a or b.
+extern "C" int dinfer_axpby(int dtype, const void* a, int64_t ld_a, float alpha, const void* b, int64_t ld_b, float beta,
+                            void* out, int64_t ld_out, int64_t rows, int64_t cols, hipStream_t stream) {
+  if (rows <= 0 || cols <= 0) return OK;
+  if (rows > 65535) return ERR_BAD_SHAPE;
+  const dim3 grid((unsigned)((cols + 255) / 256 < 64 ? (cols + 255) / 256 : 64), (unsigned)rows);
+  DINFER_DISPATCH_DTYPE(dtype, {
+    axpby_kernel<S><<<grid, 256, 0, stream>>>((const S*)a, ld_a, alpha, (const S*)b, ld_b, beta, (S*)out, ld_out, cols);
+  });
+  return launch_status();
+}
+
+// x[t, i] += a[t, i] + vec[i] (a and vec may each be null); x, a and vec each float or bf16.
+extern "C" int dinfer_add_rows(void* x, int x_dtype, int64_t ld_x, const void* a, int a_dtype, int64_t ld_a,
+                               const void* vec, int vec_dtype, int64_t rows, int64_t width, hipStream_t stream) {
+  if (rows <= 0 || width <= 0) return OK;
+  if (rows > 65535) return ERR_BAD_SHAPE;
+  const dim3 grid((unsigned)((width + 255) / 256 < 64 ? (width + 255) / 256 : 64), (unsigned)rows);
+#define ADD_ROWS(SX, SA, SV)                                                                                     \
+  add_rows_kernel<SX, SA, SV><<<grid, 256, 0, stream>>>((SX*)x, ld_x, (const SA*)a, ld_a, (const SV*)vec, width)
+  const int key = (x_dtype == DT_F32 ? 4 : 0) | (a_dtype == DT_F32 ? 2 : 0) | (vec_dtype == DT_F32 ? 1 : 0);
+  for (int dt : {x_dtype, a_dtype, vec_dtype})
+    if (dt != DT_F32 && dt != DT_BF16) return ERR_BAD_DTYPE;
+  switch (key) {
+    case 0: ADD_ROWS(bf16, bf16, bf16); break;
+    case 1: ADD_ROWS(bf16, bf16, float); break;
+    case 2: ADD_ROWS(bf16, float, bf16); break;
+    case 3: ADD_ROWS(bf16, float, float); break;
+    case 4: ADD_ROWS(float, bf16, bf16); break;
+    case 5: ADD_ROWS(float, bf16, float); break;
+    case 6: ADD_ROWS(float, float, bf16); break;
+    default: ADD_ROWS(float, float, float); break;
+  }
+#undef ADD_ROWS
+  return launch_status();
+}

@@ -103,6 +103,9 @@ void* dh_cache_create(int32_t n_groups, const int32_t* page_sizes, const int32_t
     return out;
 }
 void dh_cache_destroy(void* cache) { delete C(cache); }
+int32_t dh_cache_set_keep_first(void* cache, int32_t group, int32_t n) {
+    return guarded([&] { C(cache)->set_keep_first(group, n); return 0; });
+}
 int32_t dh_cache_has(void* cache, int64_t rid) { return C(cache)->has(rid) ? 1 : 0; }
 int32_t dh_cache_can_admit(void* cache) { return C(cache)->can_admit() ? 1 : 0; }
 int32_t dh_cache_admit(void* cache, int64_t rid) {

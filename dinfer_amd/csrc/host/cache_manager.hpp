@@ -44,6 +44,7 @@ struct GroupSpec {
     int page_size;
     int num_blocks;
     int window;  // < 0: every key of the request is kept; W >= 1: the last W keys
+    int keep_first = 0;  // with a window: the first keep_first keys stay visible, their pages are never given back
 };
 
 class CacheManager {
@@ -133,8 +134,14 @@ public:
         return true;
     }
 
+    void set_keep_first(int g, int n) {
+        if (g < 0 || g >= static_cast<int>(groups_.size()) || n < 0) throw Error(ERR_VALUE, "no such group, or a negative count");
+        if (!reqs_.empty()) throw Error(ERR_VALUE, "the kept keys of a group are set before any request is admitted");
+        groups_[g].keep_first = n;
+    }
+
     // After a step: frees the pages of window groups that the token at position num_computed and
-    // all later ones cannot see. Returns how many were freed.
+    // all later ones cannot see (the pages of the group's kept first keys stay). Returns how many were freed.
     int release_passed(int64_t rid, int64_t num_computed) {
         Req& r = find(rid);
         int freed = 0;
@@ -144,13 +151,14 @@ public:
             std::vector<int32_t>& tab = r.tables[g];
             int64_t first_key = std::max<int64_t>(0, num_computed - gs.window + 1);
             size_t first = std::min<size_t>(static_cast<size_t>(first_key / gs.page_size), tab.size());
+            size_t kept = static_cast<size_t>((gs.keep_first + gs.page_size - 1) / gs.page_size);
             scratch_.clear();
-            for (size_t i = 0; i < first; ++i)
+            for (size_t i = kept; i < first; ++i)
                 if (tab[i] >= 0) scratch_.push_back(tab[i]);
             if (scratch_.empty()) continue;
             pools_[g].free(scratch_.data(), static_cast<int>(scratch_.size()));
             freed += static_cast<int>(scratch_.size());
-            for (size_t i = 0; i < first; ++i) tab[i] = -1;
+            for (size_t i = kept; i < first; ++i) tab[i] = -1;
         }
         return freed;
     }

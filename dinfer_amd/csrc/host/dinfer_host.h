@@ -29,6 +29,8 @@ int32_t dh_pool_check(void* pool);
 void* dh_cache_create(int32_t n_groups, const int32_t* page_sizes, const int32_t* num_blocks, const int32_t* windows,
                       int32_t max_seqs, int32_t prefix_cache);
 void dh_cache_destroy(void* cache);
+/* with a window: the pages of the group's first n keys are never given back while the request lives */
+int32_t dh_cache_set_keep_first(void* cache, int32_t group, int32_t n);
 int32_t dh_cache_has(void* cache, int64_t rid);
 int32_t dh_cache_can_admit(void* cache);
 int32_t dh_cache_admit(void* cache, int64_t rid);                         /* the state slot */

@@ -295,3 +295,72 @@ extern "C" int dinfer_layernorm(const void* x, int x_dtype, void* residual, int 
       x, x_dtype, residual, res_dtype, rows, w, b, param_dtype, out, out_dtype, width, ld_x, ld_res, eps);
   return launch_status();
 }
+
+// A residual stream between norms on both sides of every sublayer:
+//   stream[s] += mult * branch[s] / sqrt(mean(branch[s]^2) + eps_b) * (wb + off_b)       (with a branch)
+//   out[r]     = stream[s] / sqrt(mean(stream[s]^2) + eps) * (w + off)                   (with an out)
+// s = rows[r] where rows are given (the model's last norm, on the rows whose logits are wanted), else r. Branch,
+// stream, gains and out each have a storage type of their own (a float stream beside bf16 branches and outputs);
+// sums, divisions and the addition are float, each stored value is rounded once. The row waits in LDS.
+namespace {
+
+__global__ void __launch_bounds__(256) rmsnorm_stream_kernel(const void* __restrict__ branch, int b_dt, int64_t ld_b,
+                                                             const void* __restrict__ wb, float eps_b, float off_b,
+                                                             float mult, void* __restrict__ stream, int s_dt,
+                                                             int64_t ld_s, const int32_t* __restrict__ rows,
+                                                             const void* __restrict__ w, int p_dt,
+                                                             void* __restrict__ out, int o_dt, float eps, float off,
+                                                             int64_t width) {
+  extern __shared__ float row[];
+  __shared__ float red[16];
+  const int64_t r = blockIdx.x;
+  const int64_t s = rows ? (int64_t)rows[r] : r;
+  float ss = 0.f;
+  if (branch) {
+    for (int64_t i = threadIdx.x; i < width; i += blockDim.x) {
+      const float v = ld_any(branch, s * ld_b + i, b_dt);
+      row[i] = v;
+      ss = add_square(ss, v);
+    }
+    const float inv_b = 1.f / sqrtf(block_sum(ss, red) / (float)width + eps_b);
+    ss = 0.f;
+    for (int64_t i = threadIdx.x; i < width; i += blockDim.x) {   // each thread re-reads what it wrote itself
+      const float y = row[i] * inv_b * (ld_any(wb, i, p_dt) + off_b);
+      const float x = round_any(__builtin_fmaf(mult, y, ld_any(stream, s * ld_s + i, s_dt)), s_dt);
+      st_any(stream, s * ld_s + i, s_dt, x);
+      row[i] = x;
+      ss = add_square(ss, x);
+    }
+  } else {
+    for (int64_t i = threadIdx.x; i < width; i += blockDim.x) {
+      const float x = ld_any(stream, s * ld_s + i, s_dt);
+      row[i] = x;
+      ss = add_square(ss, x);
+    }
+  }
+  if (!out) return;
+  const float inv = 1.f / sqrtf(block_sum(ss, red) / (float)width + eps);
+  for (int64_t i = threadIdx.x; i < width; i += blockDim.x)
+    st_any(out, r * width + i, o_dt, row[i] * inv * (ld_any(w, i, p_dt) + off));
+}
+
+}  // namespace
+
+// branch (may be null) [*, ld_b]; stream [*, ld_s], updated in place where a branch is given; out (may be null) dense
+// [n_rows, width]; wb and w share the storage type param_dtype. Width up to 16,384.
+extern "C" int dinfer_rmsnorm_stream(const void* branch, int branch_dtype, int64_t ld_b, const void* wb, float eps_b,
+                                     float off_b, float mult, void* stream_, int stream_dtype, int64_t ld_s,
+                                     const int32_t* rows, const void* w, int param_dtype, void* out, int out_dtype,
+                                     float eps, float off, int64_t n_rows, int64_t width, hipStream_t stream) {
+  if (n_rows <= 0) return OK;
+  if (width <= 0 || ld_s < width || (branch && (ld_b < width || !wb)) || (out && !w) || (!branch && !out) ||
+      n_rows > 0x7fffffff)
+    return ERR_BAD_SHAPE;
+  for (int dt : {branch_dtype, stream_dtype, param_dtype, out_dtype})
+    if (dt != DT_F32 && dt != DT_BF16) return ERR_BAD_DTYPE;
+  if (width > 16384) return ERR_UNSUPPORTED;
+  rmsnorm_stream_kernel<<<(unsigned)n_rows, 256, (size_t)width * sizeof(float), stream>>>(
+      branch, branch_dtype, ld_b, wb, eps_b, off_b, mult, stream_, stream_dtype, ld_s, rows, w, param_dtype, out,
+      out_dtype, eps, off, width);
+  return launch_status();
+}

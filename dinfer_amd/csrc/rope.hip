@@ -8,7 +8,8 @@
 //          angles of the token's position, all in float, one rounding.
 //          q is written back in place; k goes to the cache only, or, where no
 //          slot mapping is given (nothing is cached), back in place like q.
-//   v:     copied to the cache unchanged.
+//   v:     copied to the cache unchanged. Its heads may have a size of their own (v_dim); without value pages
+//          (a layer whose values are its keys) nothing is copied.
 //
 // Cache pages (chosen for MFMA operand loads on gfx950: both operands of
 // Q.K^T and P.V want 8 consecutive elements of the contraction dimension):
@@ -43,7 +44,7 @@ __global__ void __launch_bounds__(WAVES * 64) qkv_post_kernel(
     S* __restrict__ qkv, int64_t ld, int64_t q_off, int64_t k_off, int64_t v_off, const void* __restrict__ wq,
     const void* __restrict__ wk, int wf32, float eps, float w_offset, const int32_t* __restrict__ pos,
     const float* __restrict__ cos_sin, int rot, int style, S* __restrict__ k_cache, S* __restrict__ v_cache,
-    const int64_t* __restrict__ slots, int H, int Hkv, int D, int page) {
+    const int64_t* __restrict__ slots, int H, int Hkv, int D, int page, int Dv) {
   __shared__ float xs[WAVES][MAX_D];
   const int64_t t = blockIdx.x;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -57,11 +58,11 @@ __global__ void __launch_bounds__(WAVES * 64) qkv_post_kernel(
   const int64_t blk = slot >= 0 ? slot / page : 0;
   const int off = slot >= 0 ? (int)(slot % page) : 0;
 
-  if (is_v && slot >= 0) {  // a v head: cache copy only
+  if (is_v && slot >= 0 && v_cache) {  // a v head: cache copy only
     const int hk = item - H - Hkv;
-    const S* vs = row + v_off + (int64_t)hk * D;
-    S* vd = v_cache + ((blk * Hkv + hk) * (int64_t)D) * page + off;
-    for (int d = lane; d < D; d += 64) vd[(int64_t)d * page] = vs[d];
+    const S* vs = row + v_off + (int64_t)hk * Dv;
+    S* vd = v_cache + ((blk * Hkv + hk) * (int64_t)Dv) * page + off;
+    for (int d = lane; d < Dv; d += 64) vd[(int64_t)d * page] = vs[d];
   }
 
   const int hk = item - H;
@@ -388,7 +389,10 @@ extern "C" int dinfer_qkv_post(int dtype, void* qkv, int64_t tokens, int64_t ld,
                                int64_t v_off, const void* q_gain, const void* k_gain, int w_f32, float eps,
                                float w_offset, const int32_t* positions, const float* cos_sin, int rotary_dim,
                                int style, void* k_cache, void* v_cache, const int64_t* slot_mapping, int heads,
-                               int kv_heads, int head_dim, int page_size, int token_runs, hipStream_t stream) {
+                               int kv_heads, int head_dim, int page_size, int token_runs, int v_dim,
+                               hipStream_t stream) {
+  // v_dim: the size of a value head, 0 for head_dim. v_cache may be null beside a k_cache (values are not stored).
+  if (v_dim <= 0) v_dim = head_dim;
   // token_runs: the tokens come in runs of consecutive positions of a request (prompt portions), so
   // that gathering 8 tokens' values into 16-byte rows of the transposed V pages pays
   if (tokens <= 0) return OK;
@@ -399,7 +403,8 @@ extern "C" int dinfer_qkv_post(int dtype, void* qkv, int64_t tokens, int64_t ld,
   if ((q_gain == nullptr) != (k_gain == nullptr)) return ERR_BAD_SHAPE;
   const int items = heads + 2 * kv_heads;
   const dim3 grid((unsigned)tokens, (unsigned)((items + WAVES - 1) / WAVES));
-  const bool whole_head_neox = style == 0 && head_dim % 2 == 0 && (!cos_sin || rotary_dim == head_dim);
+  const bool whole_head_neox = style == 0 && head_dim % 2 == 0 && (!cos_sin || rotary_dim == head_dim) &&
+                               v_dim == head_dim && (v_cache || !slot_mapping);
   const bool vec_ok = dtype == DT_BF16 && (head_dim == 64 || head_dim == 128 || head_dim == 256) && ld % 8 == 0 &&
                       q_off % 8 == 0 && k_off % 8 == 0 && v_off % 8 == 0 && ((uintptr_t)qkv % 16) == 0 &&
                       ((uintptr_t)q_gain % 16) == 0 && ((uintptr_t)k_gain % 16) == 0 && ((uintptr_t)cos_sin % 16) == 0 &&
@@ -445,7 +450,7 @@ extern "C" int dinfer_qkv_post(int dtype, void* qkv, int64_t tokens, int64_t ld,
     qkv_post_kernel<S><<<grid, WAVES * 64, 0, stream>>>((S*)qkv, ld, q_off, k_off, v_off, q_gain, k_gain, w_f32, eps,
                                                         w_offset, positions, cos_sin, rotary_dim, style, (S*)k_cache,
                                                         (S*)v_cache, slot_mapping, heads, kv_heads, head_dim,
-                                                        page_size);
+                                                        page_size, v_dim);
   });
   return launch_status();
 }

@@ -185,7 +185,9 @@ class ModelRunner:
             raise RuntimeError(f"one request of max_model_len {opt.max_model_len} needs {self.max_blocks_per_seq} "
                                f"pages, the pool has {num_blocks}")
         self.num_blocks = int(num_blocks)
-        self.group_specs = [GroupSpec(self.page_size, self.num_blocks, window=w) for w in windows]
+        kept = {keys.index(n.group_key()): n.keep_first for n in needs if n is not None and n.group_key() is not None}
+        self.group_specs = [GroupSpec(self.page_size, self.num_blocks, window=w, keep_first=kept.get(g, 0) if w else 0)
+                            for g, w in enumerate(windows)]
         prefix = opt.enable_prefix_caching
         rebuilt_from_tokens = all(n.recomputable for n in needs if n is not None)
         if prefix is None:

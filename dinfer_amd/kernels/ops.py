@@ -192,6 +192,138 @@ def layernorm(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, 
     return out
 
 
+def rmsnorm_stream(stream: torch.Tensor, n_rows: int, *, branch: torch.Tensor | None = None,
+                   branch_weight: torch.Tensor | None = None, branch_eps: float = 0.0, branch_offset: float = 0.0,
+                   mult: float = 1.0, out: torch.Tensor | None = None, weight: torch.Tensor | None = None,
+                   eps: float = 0.0, offset: float = 0.0, rows: torch.Tensor | None = None) -> torch.Tensor | None:
+    """With a branch: stream += mult * rmsnorm(branch) * (branch_weight + branch_offset), in place. With an out:
+    out[r] = rmsnorm(stream[src r]) * (weight + offset). rows: int32 source rows (both steps act on those rows only).
+    Stream, branch and out may each be float32 or bfloat16; the two weights share a type."""
+    _need_gpu(stream, branch, branch_weight, out, weight, rows)
+    width = stream.shape[1]
+    params = [t for t in (branch_weight, weight) if t is not None]
+    assert params and all(t.dtype == params[0].dtype and t.numel() == width and t.is_contiguous() for t in params)
+    if branch is not None:
+        assert branch_weight is not None and branch.shape[1] == width
+    if out is not None:
+        assert weight is not None and out.is_contiguous() and out.shape[1] == width and out.shape[0] >= n_rows
+    if rows is not None:
+        assert rows.dtype == torch.int32 and rows.is_contiguous() and rows.numel() >= n_rows
+    else:
+        assert stream.shape[0] >= n_rows and (branch is None or branch.shape[0] >= n_rows)
+    lib.call("dinfer_rmsnorm_stream", _ptr(branch), dtype_code(branch.dtype) if branch is not None else 0,
+             _rows(branch) if branch is not None else 0, _ptr(branch_weight), float(branch_eps), float(branch_offset),
+             float(mult), stream.data_ptr(), dtype_code(stream.dtype), _rows(stream), _ptr(rows), _ptr(weight),
+             dtype_code(params[0].dtype), _ptr(out), dtype_code(out.dtype) if out is not None else 0, float(eps),
+             float(offset), n_rows, width, _stream())
+    return out
+
+
+def axpby(a: torch.Tensor, alpha: float, b: torch.Tensor, beta: float, out: torch.Tensor, rows: int) -> torch.Tensor:
+    """out[:rows] = alpha * a[:rows] + beta * b[:rows]; out may be a or b."""
+    _need_gpu(a, b, out)
+    cols = out.shape[1]
+    assert a.shape[1] == cols and b.shape[1] == cols and a.dtype == b.dtype == out.dtype
+    assert min(a.shape[0], b.shape[0], out.shape[0]) >= rows
+    done = 0
+    while done < rows:      # (the launch takes up to 65,535 rows)
+        n = min(rows - done, 65535)
+        lib.call("dinfer_axpby", dtype_code(a.dtype), a[done:].data_ptr(), _rows(a), float(alpha), b[done:].data_ptr(),
+                 _rows(b), float(beta), out[done:].data_ptr(), _rows(out), n, cols, _stream())
+        done += n
+    return out
+
+
+def add_rows(x: torch.Tensor, rows: int, a: torch.Tensor | None = None, vec: torch.Tensor | None = None) -> None:
+    """x[:rows] += a[:rows] + vec (each optional), float arithmetic, one rounding."""
+    _need_gpu(x, a, vec)
+    width = x.shape[1]
+    assert x.shape[0] >= rows and (a is None or (a.shape[1] == width and a.shape[0] >= rows))
+    assert vec is None or (vec.numel() == width and vec.is_contiguous())
+    done = 0
+    while done < rows:
+        n = min(rows - done, 65535)
+        lib.call("dinfer_add_rows", x[done:].data_ptr(), dtype_code(x.dtype), _rows(x),
+                 a[done:].data_ptr() if a is not None else None, dtype_code(a.dtype) if a is not None else 0,
+                 _rows(a) if a is not None else 0, _ptr(vec), dtype_code(vec.dtype) if vec is not None else 0, n, width,
+                 _stream())
+        done += n
+
+
+# ---- gated delta rule ----------------------------------------------------------------------------
+DELTA_MAX_DIM = 256      # the largest key size of the recurrence kernel (a thread holds 32 rows of a column)
+DELTA_MAX_HEAD = 512     # the largest key or value size of the kernels around it
+DELTA_MAX_TAPS = 16
+
+
+def delta_work_columns(qk_heads: int, heads: int, dim: int, vdim: int) -> int:
+    """Columns of the float rows between the delta rule's kernels: q | k | v | step sizes | decays."""
+    return 2 * qk_heads * dim + heads * vdim + 2 * heads
+
+
+def delta_prep(proj: torch.Tensor, tokens: int, *, qkv_off: int, b_off: int, a_off: int, taps: torch.Tensor,
+               a_log: torch.Tensor, dt_bias: torch.Tensor, conv_state: torch.Tensor | None, state_slots: torch.Tensor,
+               cu_seqlens: torch.Tensor, seq_lens: torch.Tensor, work: torch.Tensor, num_reqs: int, qk_heads: int,
+               heads: int, dim: int, vdim: int, eps: float, q_scale: float) -> None:
+    """Short convolution (over the step's rows and the request's stored inputs), silu, unit q and k, step sizes and
+    decays: proj [T, *] -> work [T, delta_work_columns] float32."""
+    _need_gpu(proj, taps, a_log, dt_bias, conv_state, state_slots, cu_seqlens, seq_lens, work)
+    C = 2 * qk_heads * dim + heads * vdim
+    K = taps.shape[1]
+    assert taps.dtype == torch.float32 and tuple(taps.shape) == (C, K) and taps.is_contiguous()
+    assert a_log.dtype == dt_bias.dtype == torch.float32 and a_log.numel() == heads == dt_bias.numel()
+    assert work.dtype == torch.float32 and work.shape[0] >= tokens and work.shape[1] >= C + 2 * heads
+    assert proj.shape[0] >= tokens and max(qkv_off + C, b_off + heads, a_off + heads) <= proj.shape[1]
+    if K > 1:
+        assert conv_state is not None and conv_state.dtype == proj.dtype and conv_state.is_contiguous()
+        assert tuple(conv_state.shape[1:]) == (C, K - 1)
+    lib.call("dinfer_delta_prep", dtype_code(proj.dtype), proj.data_ptr(), _rows(proj), qkv_off, b_off, a_off,
+             taps.data_ptr(), a_log.data_ptr(), dt_bias.data_ptr(), _ptr(conv_state) if K > 1 else None,
+             state_slots.data_ptr(), cu_seqlens.data_ptr(), seq_lens.data_ptr(), work.data_ptr(), _rows(work), num_reqs,
+             tokens, qk_heads, heads, dim, vdim, K, float(eps), float(q_scale), _stream())
+
+
+def delta_conv_update(proj: torch.Tensor, *, qkv_off: int, conv_state: torch.Tensor, state_slots: torch.Tensor,
+                      cu_seqlens: torch.Tensor, seq_lens: torch.Tensor, num_reqs: int) -> None:
+    """The step's last taps - 1 inputs a channel become the request's stored inputs (run after delta_prep)."""
+    _need_gpu(proj, conv_state, state_slots, cu_seqlens, seq_lens)
+    _, C, K1 = conv_state.shape
+    if K1 == 0:
+        return
+    assert conv_state.dtype == proj.dtype and conv_state.is_contiguous() and qkv_off + C <= proj.shape[1]
+    lib.call("dinfer_delta_conv_update", dtype_code(proj.dtype), proj.data_ptr(), _rows(proj), qkv_off,
+             conv_state.data_ptr(), state_slots.data_ptr(), cu_seqlens.data_ptr(), seq_lens.data_ptr(), num_reqs, C,
+             K1 + 1, _stream())
+
+
+def delta_recurrence(work: torch.Tensor, state: torch.Tensor, out: torch.Tensor, *, state_slots: torch.Tensor,
+                     cu_seqlens: torch.Tensor, seq_lens: torch.Tensor, num_reqs: int, qk_heads: int, heads: int,
+                     dim: int, vdim: int) -> torch.Tensor:
+    """The recurrence over each request's rows of the step. state [slots, heads, vdim, dim] float32 (a head's matrix
+    transposed), updated in place; out [T, heads * vdim] float32."""
+    _need_gpu(work, state, out, state_slots, cu_seqlens, seq_lens)
+    assert work.dtype == state.dtype == out.dtype == torch.float32 and state.is_contiguous()
+    assert tuple(state.shape[1:]) == (heads, vdim, dim) and out.shape[1] >= heads * vdim
+    assert work.shape[1] >= delta_work_columns(qk_heads, heads, dim, vdim)
+    lib.call("dinfer_delta_recurrence", work.data_ptr(), _rows(work), state.data_ptr(), state_slots.data_ptr(),
+             cu_seqlens.data_ptr(), seq_lens.data_ptr(), out.data_ptr(), _rows(out), num_reqs, qk_heads, heads, dim, vdim,
+             _stream())
+    return out
+
+
+def delta_out(o: torch.Tensor, proj: torch.Tensor, g_off: int, weight: torch.Tensor, out: torch.Tensor, tokens: int, *,
+              heads: int, vdim: int, eps: float, col_off: int = 0, out_scale: float = 1.0) -> torch.Tensor:
+    """out[t, col_off + h vdim + d] = o / rms_d(o) * weight[d] * silu(proj[t, g_off + h vdim + d]) * out_scale."""
+    _need_gpu(o, proj, weight, out)
+    assert o.dtype == torch.float32 and weight.dtype == torch.float32 and weight.numel() == vdim
+    assert proj.dtype == out.dtype and min(o.shape[0], proj.shape[0], out.shape[0]) >= tokens
+    assert g_off + heads * vdim <= proj.shape[1] and col_off + heads * vdim <= out.shape[1]
+    lib.call("dinfer_delta_out", dtype_code(out.dtype), o.data_ptr(), _rows(o), proj.data_ptr(), _rows(proj), g_off,
+             weight.data_ptr(), out.data_ptr(), _rows(out), col_off, tokens, heads, vdim, float(eps), float(out_scale),
+             _stream())
+    return out
+
+
 # ---- latent attention ----------------------------------------------------------------------------
 # Cache pages [blocks, page, R + dr]: one row a token, the normed latent and then the rotated shared key part.
 LATENT_MAX_RANK = 1024   # the largest latent the attention kernels hold in registers
@@ -407,18 +539,22 @@ def k_cache_rows(pages: torch.Tensor) -> torch.Tensor:
     return pages.permute(0, 1, 3, 2, 4).reshape(nb, hkv, page, pieces * 8)
 
 
-def _check_pages(k_cache, v_cache, kv_heads, head_dim, page_size) -> None:
+def _check_pages(k_cache, v_cache, kv_heads, head_dim, page_size, v_dim=None) -> None:
     nb = k_cache.shape[0]
     assert tuple(k_cache.shape) == k_cache_shape(nb, kv_heads, page_size, head_dim) and k_cache.is_contiguous()
-    assert tuple(v_cache.shape) == v_cache_shape(nb, kv_heads, page_size, head_dim) and v_cache.is_contiguous()
+    if v_cache is not None:
+        vd = head_dim if v_dim is None else v_dim
+        assert tuple(v_cache.shape) == v_cache_shape(nb, kv_heads, page_size, vd) and v_cache.is_contiguous()
 
 
 def qkv_post(qkv: torch.Tensor, tokens: int, *, heads: int, kv_heads: int, head_dim: int, q_off: int, k_off: int,
              v_off: int, q_gain: torch.Tensor | None, k_gain: torch.Tensor | None, eps: float, gain_offset: float,
              positions: torch.Tensor, cos_sin: torch.Tensor | None, rotary_dim: int, rope_style: int,
              k_cache: torch.Tensor | None, v_cache: torch.Tensor | None, slot_mapping: torch.Tensor | None,
-             page_size: int, token_runs: bool = True) -> None:
+             page_size: int, token_runs: bool = True, v_dim: int | None = None) -> None:
     """Per-head q/k norm, rotation, q written back in place, k and v written to the cache pages.
+    v_dim: the size of a value head where it is not head_dim. v_cache None beside a k_cache: the values are not stored
+    (a layer whose values are its keys reads them from the key pages).
 
     k_cache and v_cache in the page layouts above; slot_mapping int64 [T] (None: nothing is written
     to the cache and k is written back in place, as q is). token_runs: the tokens come in runs of consecutive positions (prompt portions, not
@@ -427,7 +563,8 @@ def qkv_post(qkv: torch.Tensor, tokens: int, *, heads: int, kv_heads: int, head_
     _need_gpu(qkv, q_gain, k_gain, positions, cos_sin, k_cache, v_cache, slot_mapping)
     ld = _rows(qkv)
     assert qkv.shape[0] >= tokens
-    assert max(q_off + heads * head_dim, k_off + kv_heads * head_dim, v_off + kv_heads * head_dim) <= qkv.shape[1]
+    vd = head_dim if v_dim is None else v_dim
+    assert max(q_off + heads * head_dim, k_off + kv_heads * head_dim, v_off + kv_heads * vd) <= qkv.shape[1]
     assert positions.dtype == torch.int32 and positions.numel() >= tokens
     wf32 = 0
     if q_gain is not None:
@@ -438,13 +575,37 @@ def qkv_post(qkv: torch.Tensor, tokens: int, *, heads: int, kv_heads: int, head_
         assert cos_sin.dtype == torch.float32 and cos_sin.is_contiguous() and cos_sin.shape[1] == rotary_dim
     if slot_mapping is not None:
         assert slot_mapping.dtype == torch.int64 and slot_mapping.numel() >= tokens
-        assert k_cache is not None and v_cache is not None
-        _check_pages(k_cache, v_cache, kv_heads, head_dim, page_size)
-        assert k_cache.dtype == qkv.dtype and v_cache.dtype == qkv.dtype
+        assert k_cache is not None
+        _check_pages(k_cache, v_cache, kv_heads, head_dim, page_size, vd)
+        assert k_cache.dtype == qkv.dtype and (v_cache is None or v_cache.dtype == qkv.dtype)
     lib.call("dinfer_qkv_post", dtype_code(qkv.dtype), qkv.data_ptr(), tokens, ld, q_off, k_off, v_off,
              _ptr(q_gain), _ptr(k_gain), wf32, float(eps), float(gain_offset), positions.data_ptr(), _ptr(cos_sin),
              rotary_dim, rope_style, _ptr(k_cache), _ptr(v_cache), _ptr(slot_mapping), heads, kv_heads, head_dim,
-             page_size, int(token_runs), _stream())
+             page_size, int(token_runs), vd, _stream())
+
+
+def attn_paged_ext(q: torch.Tensor, out: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor | None,
+                   block_table: torch.Tensor, cu_seqlens: torch.Tensor, seq_lens: torch.Tensor, num_reqs: int,
+                   tokens: int, *, scale: float, window: int, heads: int, kv_heads: int, head_dim: int, page_size: int,
+                   v_dim: int | None = None, keep_first: int = 0, sinks: torch.Tensor | None = None,
+                   slope_exp: float = 0.0, out_scale: float = 1.0) -> torch.Tensor:
+    """The plain kernel with its options: keys j < keep_first stay visible behind the window; sinks (float32 [heads])
+    join the softmax's denominator; slope_exp E takes 2^(-E (h + 1) / heads) * distance off the scores; values of size
+    v_dim, or read from the key pages (v_cache None); the output times out_scale. Any storage type."""
+    _need_gpu(q, out, k_cache, v_cache, block_table, cu_seqlens, seq_lens, sinks)
+    vd = head_dim if v_dim is None else v_dim
+    _check_pages(k_cache, v_cache, kv_heads, head_dim, page_size, vd)
+    assert q.dtype == out.dtype == k_cache.dtype and q.shape[0] >= tokens and out.shape[0] >= tokens
+    assert q.shape[1] >= heads * head_dim and out.shape[1] >= heads * vd
+    assert block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.shape[0] >= num_reqs
+    assert cu_seqlens.dtype == torch.int32 and seq_lens.dtype == torch.int32
+    if sinks is not None:
+        assert sinks.dtype == torch.float32 and sinks.numel() == heads and sinks.is_contiguous()
+    lib.call("dinfer_attn_paged_ext", dtype_code(q.dtype), q.data_ptr(), _rows(q), out.data_ptr(), _rows(out),
+             k_cache.data_ptr(), _ptr(v_cache), block_table.data_ptr(), block_table.shape[1], cu_seqlens.data_ptr(),
+             seq_lens.data_ptr(), num_reqs, tokens, float(scale), int(window), int(keep_first), _ptr(sinks),
+             float(slope_exp), heads, kv_heads, head_dim, vd, page_size, float(out_scale), _stream())
+    return out
 
 
 def attn_paged_ref(q: torch.Tensor, out: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,

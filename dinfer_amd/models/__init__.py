@@ -1,1 +1,1 @@
-from . import kudurax, qwen3  # noqa: F401  (register the built-in architectures)
+from . import karopel, kudurax, qwen3  # noqa: F401  (register the built-in architectures)

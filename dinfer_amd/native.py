@@ -59,6 +59,7 @@ _SIGNATURES = {
     "dh_cache_lookup": (_L, [_P, _L, _P, _L]),
     "dh_cache_commit": (_I, [_P, _L, _P, _L]),
     "dh_cache_destroy": (None, [_P]),
+    "dh_cache_set_keep_first": (_I, [_P, _I, _I]),
     "dh_cache_has": (_I, [_P, _L]),
     "dh_cache_can_admit": (_I, [_P]),
     "dh_cache_admit": (_I, [_P, _L]),

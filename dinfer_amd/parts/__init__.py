@@ -1,5 +1,5 @@
-from . import attention, block, latent_attention, mlp, moe, norm, position, stream_ops  # noqa: F401  (register the built-in parts)
+from . import attention, block, delta_rule, joined, latent_attention, mlp, moe, norm, position, stream_ops  # noqa: F401  (register the built-in parts)
 from .base import Block, BuildContext, CacheView, Carried, FeedForward, Into, Mixer, Norm, Part, PositionEncoding, Workspace
 from .model import DecoderModel, expected_tensors
 from .registry import BLOCKS, FEED_FORWARDS, MIXERS, NORMS, POSITION_ENCODINGS, STREAM_OPS, Registry
-from .spec import CacheSpec, KVSpec, LatentSpec, LayerSpec, ModelSpec, PartSpec, RunEntry, StateSpec, TensorSpec, part
+from .spec import CacheSpec, DeltaStateSpec, JoinedSpec, KVSpec, LatentSpec, LayerSpec, ModelSpec, PartSpec, RunEntry, StateSpec, TensorSpec, part

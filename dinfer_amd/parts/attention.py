@@ -4,6 +4,13 @@ norm, a position encoding and an optional sliding window.
 Order of operations (models/qwen3/src/model.rs:199-315): fused q|k|v projection ->
 per-head norm of q and k -> rotation -> k, v into the cache pages -> causal
 attention over the pages (scale given, default head_dim^-0.5) -> output projection.
+
+Options, each a constructor parameter that is off by default: values of a size of their own (`v_dim`); the first
+`keep_first` keys staying visible behind the window; a learned sink a head in the softmax's denominator (`sink`, a
+tensor [heads]); a bias that takes 2^(-slope_exp (h + 1) / heads) times the distance off the scores (`slope_exp`);
+values that are the keys (`values_are_keys`: no value projection, no value pages); the output multiplied by
+`out_scale`; tensor names (`names`). A layer that uses any of the first five runs the plain kernel with options
+(csrc/attention_ref.hip) for prompt portions and single rows alike; the matrix-core kernels serve the others.
 """
 from __future__ import annotations
 
@@ -23,8 +30,13 @@ class Attention(Mixer):
     capturable = True      # every kernel reads tokens, positions, slots, tables and lengths from the batch's device buffers
     capturable_portions = True   # the choice of kernels follows the step's counts alone
 
+    NAMES = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight",
+             "q_norm": "q_norm.", "k_norm": "k_norm.", "sink": "sinks"}
+
     def __init__(self, hidden: int, heads: int, kv_heads: int, head_dim: int, position: PartSpec,
-                 qk_norm: PartSpec | None = None, window: int | None = None, scale: float | None = None):
+                 qk_norm: PartSpec | None = None, window: int | None = None, scale: float | None = None,
+                 v_dim: int | None = None, keep_first: int = 0, sink: bool = False, slope_exp: float = 0.0,
+                 values_are_keys: bool = False, out_scale: float = 1.0, names: dict | None = None):
         if heads % kv_heads:
             raise ValueError(f"heads {heads} not divisible by kv_heads {kv_heads}")
         if head_dim <= 0 or head_dim % 8 or head_dim > ops.MAX_HEAD_DIM:   # said at build, not at the first step
@@ -33,9 +45,24 @@ class Attention(Mixer):
         self.hidden, self.heads, self.kv_heads, self.head_dim = hidden, heads, kv_heads, head_dim
         self.window = window
         self.scale = float(scale) if scale is not None else head_dim ** -0.5
+        self.v_dim = head_dim if v_dim is None else int(v_dim)
+        self.keep_first, self.sink, self.slope_exp = int(keep_first), bool(sink), float(slope_exp)
+        self.values_are_keys, self.out_scale = bool(values_are_keys), float(out_scale)
+        if self.values_are_keys and self.v_dim != head_dim:
+            raise ValueError("attention: values that are the keys have the keys' size")
+        if self.keep_first < 0 or self.v_dim <= 0 or self.v_dim > ops.MAX_HEAD_DIM:
+            raise ValueError(f"attention: keep_first {keep_first} or v_dim {v_dim} out of range")
+        if self.keep_first and not window:
+            self.keep_first = 0     # without a window every key stays visible anyway
+        self.names = dict(self.NAMES, **(names or {}))
+        # what the matrix-core kernels do not do runs through the plain kernel with options
+        self.extended = bool(self.v_dim != head_dim or self.keep_first or self.sink or self.slope_exp
+                             or self.values_are_keys or self.out_scale != 1.0)
         self.q_size, self.kv_size = heads * head_dim, kv_heads * head_dim
-        self.qkv = Linear(hidden, self.q_size + 2 * self.kv_size)
-        self.o = Linear(self.q_size, hidden)
+        self.v_size = 0 if self.values_are_keys else kv_heads * self.v_dim
+        self.qkv = Linear(hidden, self.q_size + self.kv_size + self.v_size)
+        self.o = Linear(heads * self.v_dim, hidden)
+        self.sinks = None
         self.position = POSITION_ENCODINGS.get(position.kind)(head_dim=head_dim, **position.params)
         self.q_norm = self.k_norm = None
         if qk_norm is not None:
@@ -43,39 +70,71 @@ class Attention(Mixer):
             self.q_norm, self.k_norm = cls(head_dim, **qk_norm.params), cls(head_dim, **qk_norm.params)
 
     def cache_spec(self):
-        return KVSpec(self.kv_heads, self.head_dim, self.window)
+        return KVSpec(self.kv_heads, self.head_dim, self.window, v_dim=self.v_dim, keep_first=self.keep_first,
+                      values=not self.values_are_keys)
 
     def tensors(self):
-        H, D, Hd = self.hidden, self.head_dim, self.hidden
+        D, Hd, nm = self.head_dim, self.hidden, self.names
         t = {
-            "q_proj.weight": TensorSpec((self.q_size, Hd)),
-            "k_proj.weight": TensorSpec((self.kv_size, Hd)),
-            "v_proj.weight": TensorSpec((self.kv_size, Hd)),
-            "o_proj.weight": TensorSpec((Hd, self.q_size)),
+            nm["q"]: TensorSpec((self.q_size, Hd)),
+            nm["k"]: TensorSpec((self.kv_size, Hd)),
+            nm["o"]: TensorSpec((Hd, self.heads * self.v_dim)),
         }
+        if not self.values_are_keys:
+            t[nm["v"]] = TensorSpec((self.v_size, Hd))
         if self.q_norm is not None:
-            t["q_norm.weight"] = TensorSpec((D,), init="gain")
-            t["k_norm.weight"] = TensorSpec((D,), init="gain")
+            for which, norm in (("q_norm", self.q_norm), ("k_norm", self.k_norm)):
+                for n, spec in norm.tensors().items():
+                    t[nm[which] + n] = spec
+        if self.sink:
+            t[nm["sink"]] = TensorSpec((self.heads,))
         for n, spec in self.position.tensors().items():   # an encoding with parameters of its own (rotations have none)
             t["position." + n] = spec
         return t
 
-    def load(self, get):
+    # ---- the middle part alone, for a mixer that joins several (parts/joined.py) ------------------
+    @property
+    def in_columns(self) -> int:
+        return self.q_size + self.kv_size + self.v_size
+
+    @property
+    def out_columns(self) -> int:
+        return self.heads * self.v_dim
+
+    def weight_rows(self, get) -> torch.Tensor:
         # q, k, v rows concatenated into one [(H + 2 Hkv) D, hidden] operand (model.rs:141-165)
-        self.qkv.set_weight(torch.cat([get("q_proj.weight", compute=True), get("k_proj.weight", compute=True),
-                                       get("v_proj.weight", compute=True)], dim=0))
-        self.o.set_weight(get("o_proj.weight", compute=True))
+        nm = self.names
+        rows = [get(nm["q"], compute=True), get(nm["k"], compute=True)]
+        if not self.values_are_keys:
+            rows.append(get(nm["v"], compute=True))
+        return torch.cat(rows, dim=0)
+
+    def out_weight(self, get) -> torch.Tensor:
+        return get(self.names["o"], compute=True)
+
+    def load(self, get):
+        self.qkv.set_weight(self.weight_rows(get))
+        self.o.set_weight(self.out_weight(get))
+        self.load_small(get)
+
+    def load_small(self, get):
+        nm = self.names
         if self.q_norm is not None:
-            self.q_norm.load(lambda n, **kw: get("q_norm." + n, **kw))
-            self.k_norm.load(lambda n, **kw: get("k_norm." + n, **kw))
+            self.q_norm.load(lambda n, **kw: get(nm["q_norm"] + n, **kw))
+            self.k_norm.load(lambda n, **kw: get(nm["k_norm"] + n, **kw))
+        if self.sink:
+            self.sinks = get(nm["sink"]).float().contiguous()
         self.position.load(lambda n, **kw: get("position." + n, **kw))
+
+    def bind_core(self, ctx):
+        self.page_size = ctx.page_size
+        self.position.bind(ctx)
 
     def bind(self, ctx):
         ws = ctx.workspace
-        self.page_size = ctx.page_size
-        self.position.bind(ctx)
-        self.qkv_buf = ws.buffer("qkv", self.q_size + 2 * self.kv_size)
-        self.attn_buf = ws.buffer("attn", self.q_size)
+        self.bind_core(ctx)
+        self.qkv_buf = ws.buffer("qkv", self.q_size + self.kv_size + self.v_size)
+        self.attn_buf = ws.buffer("attn", self.heads * self.v_dim)
         self.out_buf = ws.buffer("mixer_out", self.hidden)
         self.attn_ws = attn_kernels.Workspace(ctx, self.heads, self.kv_heads, self.head_dim)
 
@@ -83,6 +142,16 @@ class Attention(Mixer):
         T = batch.num_tokens
         g = cache.group
         self.qkv.forward(x, self.qkv_buf, T, scratch=True)
+        self.core(self.qkv_buf, 0, self.attn_buf, 0, batch, cache)
+        return self._project_out(T, into)
+
+    def core(self, qkv_buf, col, attn_buf, out_col, batch, cache: CacheView):
+        """Everything between the two products: q | k | v are read from column `col` of qkv_buf on, the heads'
+        outputs go to column `out_col` of attn_buf (a mixer that joins several shares one product on each side)."""
+        T = batch.num_tokens
+        g = cache.group
+        if self.extended or col or out_col:
+            return self._core_plain(qkv_buf, col, attn_buf, out_col, batch, cache)
         qn, pos = self.q_norm, self.position
         geometry = dict(heads=self.heads, kv_heads=self.kv_heads, head_dim=self.head_dim, q_off=0, k_off=self.q_size,
                         v_off=self.q_size + self.kv_size, positions=batch.positions, page_size=self.page_size)
@@ -99,7 +168,7 @@ class Attention(Mixer):
                 scale=self.scale, window=self.window or 0, heads=self.heads, kv_heads=self.kv_heads,
                 head_dim=self.head_dim, page_size=self.page_size, q_off=0, k_off=self.q_size,
                 v_off=self.q_size + self.kv_size, positions=batch.positions, cos_sin=pos.table(), **norm)
-            return self._project_out(T, into)
+            return
         if pos.fused:
             # per-head norm, rotation by the encoding's table and the cache write in one kernel
             ops.qkv_post(self.qkv_buf, T, **geometry, **norm, cos_sin=pos.table(), rotary_dim=pos.rotary_dim,
@@ -118,7 +187,27 @@ class Attention(Mixer):
             self.qkv_buf, self.attn_buf, cache.k, cache.v, batch, g, self.attn_ws, scale=self.scale,
             window=self.window or 0, heads=self.heads, kv_heads=self.kv_heads, head_dim=self.head_dim,
             page_size=self.page_size)
-        return self._project_out(T, into)
+
+    def _core_plain(self, qkv_buf, col, attn_buf, out_col, batch, cache: CacheView):
+        """Per-head norm, rotation and cache write, then the plain kernel with this layer's options."""
+        T, g = batch.num_tokens, cache.group
+        qn, pos = self.q_norm, self.position
+        if not pos.fused:
+            raise NotImplementedError("attention with options takes a rotation by a table, or none")
+        vd = self.v_dim
+        ops.qkv_post(qkv_buf, T, heads=self.heads, kv_heads=self.kv_heads, head_dim=self.head_dim, q_off=col,
+                     k_off=col + self.q_size, v_off=col + self.q_size + (0 if self.values_are_keys else self.kv_size),
+                     positions=batch.positions, page_size=self.page_size,
+                     q_gain=qn.weight if qn else None, k_gain=self.k_norm.weight if qn else None,
+                     eps=qn.eps if qn else 0.0, gain_offset=qn.weight_offset if qn else 0.0,
+                     cos_sin=pos.table(), rotary_dim=pos.rotary_dim, rope_style=pos.style,
+                     k_cache=cache.k, v_cache=cache.v, slot_mapping=batch.slot_mapping[g] if cache.owner else None,
+                     token_runs=False, v_dim=vd)
+        ops.attn_paged_ext(qkv_buf[:, col:], attn_buf[:, out_col:], cache.k, cache.v, batch.block_table[g],
+                           batch.cu_seqlens, batch.seq_lens, batch.num_reqs, T, scale=self.scale,
+                           window=self.window or 0, heads=self.heads, kv_heads=self.kv_heads, head_dim=self.head_dim,
+                           page_size=self.page_size, v_dim=vd, keep_first=self.keep_first, sinks=self.sinks,
+                           slope_exp=self.slope_exp, out_scale=self.out_scale)
 
     def _project_out(self, T, into):
         if into is not None:

@@ -160,6 +160,12 @@ class CacheView:
             if t is not None:
                 self.tensors[name] = t
 
+    def child(self, name: str) -> "CacheView":
+        """The part of a joined cache that belongs to the member `name` (JoinedSpec): same group, same owner."""
+        cut = len(name) + 1
+        return CacheView(self.group, owner=self.owner,
+                         tensors={k[cut:]: t for k, t in self.tensors.items() if k.startswith(name + ".")})
+
     def __getattr__(self, name):
         # only reached for names that are no attribute of the object: the cache's tensors, None for the usual
         # three where the entry has none of that kind

@@ -13,7 +13,7 @@ from __future__ import annotations
 
 import torch
 
-from ..kernels import gemm
+from ..kernels import gemm, ops
 from .base import Block, CacheView, Carried, Into
 from .registry import BLOCKS, FEED_FORWARDS, MIXERS, NORMS
 from .spec import LayerSpec
@@ -99,3 +99,94 @@ class PreNormBlock(Block):
         else:
             x = self.norm_post.forward(a, self.normed, T, residual=hidden)
         return self.ff.forward(x, batch, **self._into(hidden, next_norm, self.ff, T))
+
+
+@BLOCKS.register("sandwich")
+class SandwichBlock(Block):
+    """A norm before and after each sublayer, and a multiplier on what is added:
+
+        h += mult * norm_a_out(mixer(norm_a(h)));   h += mult * norm_b_out(ff(norm_b(h)))
+
+    One kernel a sublayer's end norms the branch, adds it into the stream (in the stream's own dtype, 32 bits where
+    the model says so) and norms the stream for what reads it next: this block's feed-forward, or the next block's
+    mixer (handed over as a Carried that is ready). params: mult, mixer_prefix, ff_prefix and the four norms' names.
+    All four norms are of the layer's norm kind, which must be a root-mean-square norm (`carried()` gives its gain)."""
+    carries_norms = True
+
+    def __init__(self, hidden: int, layer: LayerSpec, mult: float = 1.0, mixer_prefix: str = "mix.", ff_prefix: str = "mlp.",
+                 norm_a: str = "norm1", norm_a_out: str = "norm1b", norm_b: str = "norm2", norm_b_out: str = "norm2b"):
+        self.hidden, self.mult = hidden, float(mult)
+        self.mixer = MIXERS.get(layer.mixer.kind)(hidden=hidden, **layer.mixer.params)
+        self.ff = FEED_FORWARDS.get(layer.feed_forward.kind)(hidden=hidden, **layer.feed_forward.params)
+        if getattr(self.ff, "absent", False):
+            self.ff = None
+        ncls = NORMS.get(layer.norm.kind)
+        names = [norm_a, norm_a_out] + ([norm_b, norm_b_out] if self.ff is not None else [])
+        self.norms = [(n, ncls(hidden, **layer.norm.params)) for n in names]
+        if any(n.carried() is None for _, n in self.norms):
+            raise ValueError("the sandwich arrangement takes root-mean-square norms")
+        self.prefixes = (mixer_prefix, ff_prefix)
+
+    def _parts(self):
+        out = [(self.prefixes[0], self.mixer)] + list(self.norms)
+        if self.ff is not None:
+            out.append((self.prefixes[1], self.ff))
+        return out
+
+    @property
+    def capturable(self):
+        return all(part.capturable for _, part in self._parts())
+
+    @property
+    def capturable_portions(self):
+        return all(part.capturable and part.capturable_portions for _, part in self._parts())
+
+    def tensors(self):
+        return {p + n: s for p, part in self._parts() for n, s in part.tensors().items()}
+
+    def load(self, get):
+        for p, part in self._parts():
+            part.load(_sub(get, p))
+        for _, n in self.norms:
+            n.weight = n.weight.float().contiguous()     # (exact for a bfloat16 file) one type for all gains of a kernel
+
+    def bind(self, ctx):
+        for _, part in self._parts():
+            part.bind(ctx)
+        self.normed = ctx.workspace.buffer("normed", self.hidden)
+
+    def input_norm(self):
+        return self.norms[0][1]
+
+    def _close(self, hidden, branch, norm_out, T, then):
+        """stream += mult * norm_out(branch); then the stream normed by `then` (a norm or None) into self.normed."""
+        g, off, eps = norm_out.carried()
+        kw = {}
+        if then is not None:
+            w2, off2, eps2 = then.carried()
+            kw = dict(out=self.normed, weight=w2, eps=eps2, offset=off2)
+        return ops.rmsnorm_stream(hidden, T, branch=branch, branch_weight=g, branch_eps=eps, branch_offset=off,
+                                  mult=self.mult, **kw)
+
+    def forward(self, hidden, pending, batch, cache: CacheView, next_norm=None):
+        T = batch.num_tokens
+        if isinstance(pending, Carried):
+            x = pending.materialise()
+        else:
+            if pending is not None:      # a block of another kind left its last branch to be added
+                ops.add_rows(hidden, T, a=pending)
+            x = self.norms[0][1].forward(hidden, self.normed, T)
+        a = self.mixer.forward(x, batch, cache)
+        if next_norm is not None:     # handed on only where the kernel can apply it: a gain of the type of this block's
+            params = next_norm.carried()
+            if params is None or params[0] is None or params[0].dtype != self.norms[0][1].weight.dtype:
+                next_norm = None
+        if self.ff is None:
+            self._close(hidden, a, self.norms[1][1], T, next_norm)
+        else:
+            x = self._close(hidden, a, self.norms[1][1], T, self.norms[2][1])
+            f = self.ff.forward(x, batch)
+            self._close(hidden, f, self.norms[3][1], T, next_norm)
+        if next_norm is None:
+            return None
+        return Carried(None, None, 0, 0.0, self.hidden, next_norm, hidden, self.normed, T, ready=True)

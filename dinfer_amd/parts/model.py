@@ -25,6 +25,12 @@ def _stream_ops(spec: ModelSpec) -> list:
     return made
 
 
+def _before_ops(spec: ModelSpec) -> list:
+    """Per run entry: the part applied to the stream right before it, or None."""
+    return [None if e.before is None else STREAM_OPS.get(e.before.kind)(spec.hidden_size, **e.before.params)
+            for e in spec.run]
+
+
 def expected_tensors(spec: ModelSpec, blocks=None) -> tuple[dict[str, TensorSpec], set[str]]:
     """(name -> TensorSpec for every tensor the model reads, names that may be present or absent)."""
     blocks = blocks or _build_blocks(spec)
@@ -39,6 +45,9 @@ def expected_tensors(spec: ModelSpec, blocks=None) -> tuple[dict[str, TensorSpec
         if op is not None:
             for n, ts in op[1].tensors().items():
                 exp[op[0] + n] = ts
+    for op in _before_ops(spec):
+        if op is not None:
+            exp.update(op.tensors())      # under the names they give themselves; several entries may read one table
     optional = set()
     if spec.tie_embeddings:
         # A tied checkpoint may still ship the head; it is used when present (model.rs:487-496).
@@ -56,7 +65,10 @@ class DecoderModel:
         self.head = Linear(spec.hidden_size, spec.vocab_size)
         self.embed_post, self.logits_post = _stream_ops(spec)
         self.embed: torch.Tensor | None = None
-        self.run = [RunEntry(e.layer, i if e.cache is None else e.cache) for i, e in enumerate(spec.run)]
+        self.run = [RunEntry(e.layer, i if e.cache is None else e.cache, e.before) for i, e in enumerate(spec.run)]
+        self.before = _before_ops(spec)
+        # the embeddings as they entered the stream, kept for an entry's `before` part that adds them again
+        self.keeps_embedding = any(getattr(op, "needs_embedding", False) for op in self.before if op is not None)
         for i, e in enumerate(self.run):
             if not (0 <= e.layer < len(self.blocks)):
                 raise ValueError(f"run entry {i} names layer {e.layer}, but the model has {len(self.blocks)} layers")
@@ -97,6 +109,9 @@ class DecoderModel:
         for op in (self.embed_post, self.logits_post):
             if op is not None:
                 op[1].load(lambda n, _p=op[0], **kw: get(_p + n, **kw))
+        for op in self.before:
+            if op is not None:
+                op.load(get)
 
     # ---- cache needs ---------------------------------------------------------------------------
     def cache_needs(self) -> list:
@@ -109,6 +124,7 @@ class DecoderModel:
     def capturable(self) -> bool:
         """Whether a step of single rows may be captured once and replayed for other requests."""
         ops_ = [op[1] for op in (self.embed_post, self.logits_post) if op is not None]
+        ops_ += [op for op in self.before if op is not None]
         return (all(self.blocks[e.layer].capturable for e in self.run) and self.final_norm.capturable
                 and all(o.capturable for o in ops_))
 
@@ -125,9 +141,13 @@ class DecoderModel:
         for op in (self.embed_post, self.logits_post):
             if op is not None:
                 op[1].bind(ctx)
+        for op in self.before:
+            if op is not None:
+                op.bind(ctx)
         ws = ctx.workspace
         stream = torch.float32 if self.spec.stream_dtype == "float32" else None
         self.hidden = ws.buffer("hidden", self.spec.hidden_size, dtype=stream)
+        self.embedded = ws.buffer("embedded", self.spec.hidden_size, dtype=stream) if self.keeps_embedding else None
         self.final_normed = ws.buffer("final_normed", self.spec.hidden_size, rows=ctx.max_rows)
         self.logits = torch.empty((ctx.max_rows, self.spec.vocab_size), dtype=torch.float32, device=ctx.device)
 
@@ -139,11 +159,22 @@ class DecoderModel:
                       getattr(batch, "last_tokens", None), scale=self.spec.embed_scale)
         if self.embed_post is not None:
             self.embed_post[1].forward(self.hidden, T)
+        if self.embedded is not None:
+            self.embedded[:T].copy_(self.hidden[:T])
         pending = None
         for i, e in enumerate(self.run):
-            # the input norm of the block that runs next, if that block lets the one before carry it
             block = self.blocks[e.layer]
-            if block.carries_norms and i + 1 < len(self.run):
+            if self.before[i] is not None:
+                # the stream must be whole before something is added to it from outside the blocks
+                if isinstance(pending, Carried):
+                    pending = None
+                elif pending is not None:
+                    ops.add_rows(self.hidden, T, a=pending)
+                    pending = None
+                self.before[i].forward(self.hidden, T, embedding=self.embedded)
+            # the input norm of the block that runs next, if that block lets the one before carry it (and nothing
+            # touches the stream between the two)
+            if block.carries_norms and i + 1 < len(self.run) and self.before[i + 1] is None:
                 nxt = self.blocks[self.run[i + 1].layer].input_norm()
                 pending = block.forward(self.hidden, pending, batch, caches[i], next_norm=nxt)
             else:

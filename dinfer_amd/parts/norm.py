@@ -26,6 +26,10 @@ class RMSNorm(Norm):
         return (self.weight, self.weight_offset, self.eps)
 
     def forward(self, x, out, n_rows, *, residual=None, rows=None):
+        if residual is None and x.dtype != out.dtype:
+            # a stream kept in 32 bits, normed into the engine's dtype
+            return ops.rmsnorm_stream(x, n_rows, out=out, weight=self.weight, eps=self.eps, offset=self.weight_offset,
+                                      rows=rows)
         return ops.rmsnorm(x, self.weight, out, self.eps, n_rows, residual=residual, rows=rows,
                            weight_offset=self.weight_offset)
 

@@ -9,6 +9,10 @@ With `scaling` (factor s, original length L, fast, slow; "YaRN"): dimensions tha
 frequency, those that turn rarely are slowed by s, with a linear ramp between: for d(t) = D ln(L / (2 pi t)) / (2 ln theta),
 lo = max(floor(d(fast)), 0), hi = min(ceil(d(slow)), D - 1), r_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1), the
 frequency is f_i / s * r_i + f_i * (1 - r_i), and cos and sin are both multiplied by 0.1 ln(s) + 1.
+
+With `scaling` of kind "wavelength_bands" (factor s, original length L, low, high): by the wavelength l_i = 2 pi / f_i a
+frequency is kept (l_i < L / high), divided by s (l_i > L / low), or, between the two, blended with
+t = (L / l_i - low) / (high - low) as (1 - t) f_i / s + t f_i; cos and sin keep their size.
 """
 from __future__ import annotations
 
@@ -41,17 +45,24 @@ class Rotary(PositionEncoding):
         self.head_dim, self.theta, self.max_positions = head_dim, float(theta), max_positions
         self.rotary_dim, self.style = rd, STYLES[style]
         self.scaling = None
+        self.scaling_kind = None
         if scaling:
-            sc = {k: float(scaling[k]) for k in ("factor", "original", "fast", "slow")}
-            if not (sc["factor"] > 0 and sc["original"] > 0 and sc["fast"] > 0 and sc["slow"] > 0):
-                raise ValueError(f"rotary scaling needs positive factor, original, fast and slow, got {scaling!r}")
+            self.scaling_kind = scaling.get("kind", "ramp")
+            if self.scaling_kind not in ("ramp", "wavelength_bands"):
+                raise ValueError(f"rotary scaling kind {self.scaling_kind!r} unknown; known: 'ramp', 'wavelength_bands'")
+            keys = ("factor", "original", "fast", "slow") if self.scaling_kind == "ramp" else ("factor", "original", "low", "high")
+            sc = {k: float(scaling[k]) for k in keys}
+            if not all(v > 0 for v in sc.values()):
+                raise ValueError(f"rotary scaling needs positive {', '.join(keys)}, got {scaling!r}")
+            if self.scaling_kind == "wavelength_bands" and not sc["high"] > sc["low"]:
+                raise ValueError(f"rotary scaling by wavelength needs high > low, got {scaling!r}")
             self.scaling = sc
         self._table = None
 
     def bind(self, ctx):
         # one table for all layers with the same rotation, as long as the longest request the engine admits
         n = min(self.max_positions, ctx.max_seq_len or self.max_positions)
-        sc = tuple(sorted(self.scaling.items())) if self.scaling else None
+        sc = (self.scaling_kind,) + tuple(sorted(self.scaling.items())) if self.scaling else None
         self._table = ctx.share(("rotary", self.theta, self.rotary_dim, self.style, n, sc),
                                 lambda: self.host_table(n).to(ctx.device).contiguous())
 
@@ -64,6 +75,11 @@ class Rotary(PositionEncoding):
         if self.scaling is None:
             return freq, 1.0
         sc = self.scaling
+        if self.scaling_kind == "wavelength_bands":
+            wavelength = 2 * math.pi / freq
+            t = ((sc["original"] / wavelength - sc["low"]) / (sc["high"] - sc["low"])).clamp(0, 1)
+            # t is 0 where the wavelength exceeds original / low and 1 where it is below original / high
+            return (1 - t) * freq / sc["factor"] + t * freq, 1.0
 
         def dim_of(turns: float) -> float:     # the (fractional) pair index that makes `turns` turns within the original length
             return D * math.log(sc["original"] / (2 * math.pi * turns)) / (2 * math.log(self.theta))

@@ -50,6 +50,7 @@ class CacheSpec:
     `reset_slots` clears the slots of requests that have just been admitted.
     """
     window: int | None = None      # W: pages whose keys all lie more than W before the next token are given back
+    keep_first: int = 0            # with a window: the pages of the first keep_first keys are never given back
     recomputable: bool = True      # the contents follow from the request's tokens alone (pages may be shared and refilled)
     chunk_alignment: int = 1       # prompt portions that do not end the request must end at a multiple of this
 
@@ -81,25 +82,38 @@ class KVSpec(CacheSpec):
     """Cache need of a mixer that stores a key and a value per token and kv head.
 
     window: None keeps every key of the request; W keeps the last W keys, so
-    pages that the window has passed are given back while the request lives.
+    pages that the window has passed are given back while the request lives
+    (but for the pages of the first keep_first keys, which stay visible).
+    v_dim: the size of a value head where it differs from head_dim. values False:
+    the values are the keys and only key pages are kept.
     """
     kv_heads: int
     head_dim: int
     window: int | None = None
+    v_dim: int | None = None
+    keep_first: int = 0
+    values: bool = True
 
     def group_key(self) -> tuple:
         # Layers of equal page geometry and equal window share block tables.
-        return ("kv", self.kv_heads, self.head_dim, self.window)
+        key = ("kv", self.kv_heads, self.head_dim, self.window)
+        if self.v_dim not in (None, self.head_dim) or self.keep_first or not self.values:
+            key += (self.v_dim, self.keep_first, self.values)
+        return key
 
     def page_bytes(self, page_size, dtype):
-        return 2 * self.kv_heads * self.head_dim * page_size * _element_size(dtype)
+        per_key = self.head_dim + ((self.v_dim or self.head_dim) if self.values else 0)
+        return self.kv_heads * per_key * page_size * _element_size(dtype)
 
     def allocate(self, num_blocks, page_size, num_slots, dtype, device):
         import torch
         from ..kernels import ops
-        geometry = (num_blocks, self.kv_heads, page_size, self.head_dim)
-        return {"k": torch.empty(ops.k_cache_shape(*geometry), dtype=dtype, device=device),
-                "v": torch.empty(ops.v_cache_shape(*geometry), dtype=dtype, device=device)}
+        out = {"k": torch.empty(ops.k_cache_shape(num_blocks, self.kv_heads, page_size, self.head_dim), dtype=dtype,
+                                device=device)}
+        if self.values:
+            out["v"] = torch.empty(ops.v_cache_shape(num_blocks, self.kv_heads, page_size, self.v_dim or self.head_dim),
+                                   dtype=dtype, device=device)
+        return out
 
 
 @dataclass(frozen=True)
@@ -153,6 +167,65 @@ class StateSpec(CacheSpec):
 
 
 @dataclass(frozen=True)
+class DeltaStateSpec(CacheSpec):
+    """Cache need of a delta-rule mixer: per request one float32 matrix a head, kept transposed [heads, vdim, dim],
+    and the last taps - 1 inputs of every channel of its short convolution, in the engine's dtype."""
+    heads: int
+    dim: int
+    vdim: int
+    channels: int
+    taps: int
+    recomputable = False
+
+    def slot_bytes(self, dtype):
+        return self.heads * self.dim * self.vdim * 4 + self.channels * (self.taps - 1) * _element_size(dtype)
+
+    def allocate(self, num_blocks, page_size, num_slots, dtype, device):
+        import torch
+        return {"state": torch.zeros((num_slots, self.heads, self.vdim, self.dim), dtype=torch.float32, device=device),
+                "conv": torch.zeros((num_slots, self.channels, self.taps - 1), dtype=dtype, device=device)}
+
+    def reset_slots(self, tensors, slots):
+        tensors["state"].index_fill_(0, slots, 0)
+        tensors["conv"].index_fill_(0, slots, 0)
+
+
+class JoinedSpec(CacheSpec):
+    """The cache needs of a mixer made of several mixers, by name: member `left`'s tensor `k` becomes `left.k`
+    (CacheView.child("left") shows it as `k` again). At most one member may be paged: a run entry has one block table
+    a request."""
+
+    def __init__(self, members: dict):
+        self.members = {n: m for n, m in members.items() if m is not None}
+        paged = [m for m in self.members.values() if m.group_key() is not None]
+        if len(paged) > 1:
+            raise ValueError("a joined cache may have one paged member: a run entry has one block table a request")
+        self.paged = paged[0] if paged else None
+        self.window = self.paged.window if self.paged else None
+        self.keep_first = self.paged.keep_first if self.paged else 0
+        self.recomputable = all(m.recomputable for m in self.members.values())
+        import math
+        self.chunk_alignment = math.lcm(*(m.chunk_alignment for m in self.members.values())) if self.members else 1
+
+    def group_key(self):
+        return self.paged.group_key() if self.paged else None
+
+    def page_bytes(self, page_size, dtype):
+        return sum(m.page_bytes(page_size, dtype) for m in self.members.values())
+
+    def slot_bytes(self, dtype):
+        return sum(m.slot_bytes(dtype) for m in self.members.values())
+
+    def allocate(self, num_blocks, page_size, num_slots, dtype, device):
+        return {f"{n}.{k}": t for n, m in self.members.items()
+                for k, t in m.allocate(num_blocks, page_size, num_slots, dtype, device).items()}
+
+    def reset_slots(self, tensors, slots):
+        for n, m in self.members.items():
+            m.reset_slots({k[len(n) + 1:]: t for k, t in tensors.items() if k.startswith(n + ".")}, slots)
+
+
+@dataclass(frozen=True)
 class LayerSpec:
     """One layer: which block arrangement holds which mixer, feed-forward and norm.
 
@@ -173,10 +246,14 @@ class RunEntry:
     layer: index into ModelSpec.layers (a layer may appear more than once: its
     weights are shared). cache: index of the run entry whose cache this entry
     uses; its own index by default. An entry that names another entry's cache
-    reads it and writes nothing.
+    reads it and writes nothing. before: a PartSpec of STREAM_OPS applied to the
+    residual stream right before this entry's layer (a model that runs some of
+    its layers several times may add something at the start of each pass); its
+    tensors are read under the names it gives, without a prefix.
     """
     layer: int
     cache: int | None = None
+    before: PartSpec | None = None
 
 
 @dataclass

@@ -9,6 +9,7 @@ from __future__ import annotations
 from ..kernels import ops
 from .base import Part
 from .registry import STREAM_OPS
+from .spec import TensorSpec
 
 
 @STREAM_OPS.register("scale_softcap")
@@ -22,3 +23,28 @@ class ScaleSoftcap(Part):
 
     def forward(self, x, rows: int) -> None:
         ops.scale_softcap(x, rows, self.scale, self.softcap)
+
+
+@STREAM_OPS.register("pass_start")
+class PassStart(Part):
+    """What a model that runs a group of its layers several times adds to the stream at the start of a pass
+    (RunEntry.before): x += embeddings (where `add_embedding`: the token embeddings as they first entered the stream)
+    + table[row], with `table` [rows, width] a tensor of the weight file."""
+
+    def __init__(self, width: int, table: str, rows: int, row: int, add_embedding: bool = False):
+        if not 0 <= row < rows:
+            raise ValueError(f"pass_start: row {row} of a table of {rows}")
+        self.width, self.table, self.rows, self.row = width, table, rows, row
+        self.needs_embedding = bool(add_embedding)
+        self.vec = None
+
+    def tensors(self):
+        return {self.table: TensorSpec((self.rows, self.width))}
+
+    def load(self, get):
+        self.vec = get(self.table).float()[self.row].contiguous()
+
+    def forward(self, x, rows: int, embedding=None) -> None:
+        if self.needs_embedding and embedding is None:
+            raise RuntimeError("pass_start: the model kept no embeddings to add")
+        ops.add_rows(x, rows, a=embedding if self.needs_embedding else None, vec=self.vec)
