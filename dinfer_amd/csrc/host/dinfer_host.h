@@ -52,7 +52,7 @@ int64_t dh_cache_lookup(void* cache, int64_t rid, const int32_t* tokens, int64_t
 int32_t dh_cache_commit(void* cache, int64_t rid, const int32_t* tokens, int64_t num_computed);
 
 /* ---- the flat batch of a step, written into the caller's pinned buffer */
-#define DH_MAX_GROUPS 8
+#define DH_MAX_GROUPS 16
 typedef struct {
     int32_t n_groups, max_tokens, max_reqs, max_rows;
     int32_t* input_ids;

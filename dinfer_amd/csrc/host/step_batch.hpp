@@ -28,7 +28,7 @@
 
 namespace dinfer {
 
-constexpr int MAX_GROUPS = 8;
+constexpr int MAX_GROUPS = 16;
 
 // Addresses inside the pinned buffer and the capacities they were sized for.
 struct BatchBuffers {

@@ -9,7 +9,7 @@ from ctypes import POINTER, Structure, c_char_p, c_int32, c_int64, c_void_p
 
 from .kernels.lib import load_library
 
-MAX_GROUPS = 8
+MAX_GROUPS = 16
 _I, _L, _P = c_int32, c_int64, c_void_p
 _PI, _PL = POINTER(c_int32), POINTER(c_int64)
 

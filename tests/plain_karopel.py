@@ -210,3 +210,62 @@ def forward(tokens, w, cfg):
         streams.append(x)
     y = norm_around_zero(x, w["final.norm"], cfg["norm"]["eps"])
     return (y @ w["head"].T) * cfg["logit_scale"], streams
+
+
+def tensor_shapes(cfg):
+    """name -> shape of every tensor a model of this configuration has, written out from the design."""
+    W = cfg["width"]
+    out = {"embed": (cfg["vocab"], W), "final.norm": (W,), "head": (cfg["vocab"], W)}
+    if cfg.get("loop"):
+        out["loop.step"] = (cfg["loop"]["times"], W)
+    for i, l in enumerate(cfg["layers"]):
+        p, m = f"l{i}.", l["mixer"]
+        out[p + "norm1"] = out[p + "norm1b"] = (W,)
+        if l["type"] == "attention":
+            H, G, D, V = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+            out.update({p + "mix.q": (H * D, W), p + "mix.k": (G * D, W), p + "mix.v": (G * V, W), p + "mix.q.norm": (D,),
+                        p + "mix.k.norm": (D,), p + "mix.sink": (H,), p + "mix.o": (W, H * V)})
+        else:
+            a, r = m["left"], m["right"]
+            out.update({p + "mix.left.q": (a["heads"] * a["dim"], W), p + "mix.left.k": (a["kv_heads"] * a["dim"], W),
+                        p + "mix.left.o": (W, a["heads"] * a["dim"])})
+            H, G, D, V, K = r["heads"], r["kv_heads"], r["dim"], r["vdim"], r["conv"]
+            q = p + "mix.right."
+            out.update({q + "q": (G * D, W), q + "k": (G * D, W), q + "v": (H * V, W), q + "q.conv": (G * D, K),
+                        q + "k.conv": (G * D, K), q + "v.conv": (H * V, K), q + "b": (H, W), q + "a": (H, W),
+                        q + "A_log": (H,), q + "dt_bias": (H,), q + "g": (H * V, W), q + "norm": (V,), q + "o": (W, H * V)})
+        if l.get("mlp"):
+            ff = l["mlp"]["ff"]
+            out[p + "norm2"] = out[p + "norm2b"] = (W,)
+            out.update({p + "mlp.gate": (ff, W), p + "mlp.up": (ff, W), p + "mlp.down": (W, ff)})
+    return out
+
+
+def random_weights(cfg, seed):
+    """bfloat16 tensors of sizes that keep every mechanism awake: products of unit spread, gains around their
+    neutral value, sinks and decay parameters spread over a few units."""
+    g = torch.Generator().manual_seed(seed)
+    out = {}
+    for name, shape in tensor_shapes(cfg).items():
+        last = name.split(".")[-1]
+        x = torch.randn(shape, generator=g)
+        if name in ("embed", "loop.step"):
+            t = x * (1.0 if name == "embed" else 0.3)
+        elif last in ("norm1", "norm1b", "norm2", "norm2b") or name == "final.norm":
+            t = x * 0.15                                   # stored around zero
+        elif name.endswith("q.norm") or name.endswith("k.norm") or name.endswith("right.norm"):
+            t = 1.0 + x * 0.15
+        elif last == "sink":
+            t = x * 1.5
+        elif last in ("A_log", "dt_bias"):
+            t = x * 0.7
+        elif last == "conv":
+            t = x * 0.6
+        else:
+            t = x * (1.5 / shape[-1] ** 0.5)
+        out[name] = t.to(torch.bfloat16)
+    return out
+
+
+def as_float64(w):
+    return {k: v.to(F) for k, v in w.items()}
