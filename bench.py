@@ -5,6 +5,7 @@
                     [--prompt P] [--context C] [--workload decode|serving [--sampled]]
     python bench.py --workload closed --shape 0.6b --concurrency 8 --prompt 128 --max-tokens 128 [--num-requests N]
     python bench.py --workload kudurax [--kudurax-shape 2k|4k] [--layers 4] [--prompt 2048] [--only kudurax|qwen3]
+    python bench.py --workload karopel [--karopel-shape 2k|4k] [--layers 4] [--prompt 2048] [--only karopel|qwen3]
 
 Prints ONE JSON line. `value` is decoded tokens per second at the default batch (8), each
 request with a 2,048-token prompt in a 4,096-token context; a "step" is one decode step
@@ -226,17 +227,61 @@ def kudurax_config(shape: dict, layers: int, vocab: int) -> dict:
                 layers=out)
 
 
+# Karopel layer sizes that resemble a real model's: attention layers with grouped keys and values, a window of 1,024
+# that keeps the first four tokens, and layers in which a narrower windowed attention runs beside a gated delta rule
+# of twice as many value heads as key heads, all heads 128 wide; the Qwen3 layer of the same width beside each
+KAROPEL_SHAPES = {
+    "2k": dict(width=2048, heads=16, kv_heads=4, dim=128, window=1024, keep_first=4, left_heads=8, left_kv_heads=2,
+               left_window=512, delta_heads=16, delta_qk_heads=8, conv=4, ff=8192,
+               qwen=dict(num_attention_heads=16, num_key_value_heads=4, head_dim=128, intermediate_size=8192)),
+    "4k": dict(width=4096, heads=32, kv_heads=8, dim=128, window=1024, keep_first=4, left_heads=16, left_kv_heads=4,
+               left_window=512, delta_heads=32, delta_qk_heads=16, conv=4, ff=12288,
+               qwen=dict(num_attention_heads=32, num_key_value_heads=8, head_dim=128, intermediate_size=12288)),
+}
+
+
+def karopel_config(shape: dict, layers: int, vocab: int) -> dict:
+    """Layers in fours: attention, parallel, parallel, attention; the middle two run twice."""
+    d = shape["dim"]
+    att = dict(type="attention", mlp=dict(kind="dense", ff=shape["ff"]), mixer=dict(
+        heads=shape["heads"], kv_heads=shape["kv_heads"], dim=d, vdim=d, scale=d ** -0.5,
+        mask=dict(size=shape["window"], keep_first=shape["keep_first"]),
+        rot=dict(base=500000.0, dims=d, scaling=dict(factor=8.0, low=1.0, high=4.0, original=8192))))
+    par = dict(type="parallel", mlp=dict(kind="dense", ff=shape["ff"]), mixer=dict(
+        left=dict(heads=shape["left_heads"], kv_heads=shape["left_kv_heads"], dim=d, vdim=d, scale=d ** -0.5,
+                  mask=dict(size=shape["left_window"])),
+        right=dict(heads=shape["delta_heads"], kv_heads=shape["delta_qk_heads"], dim=d, vdim=d, conv=shape["conv"]),
+        left_scale=0.5, right_scale=0.5))
+    return dict(architecture="Karopel", vocab=vocab, width=shape["width"], residual_mult=0.5, logit_scale=1.0,
+                norm=dict(eps=1e-6), loop=None, layers=[par if i % 4 in (1, 2) else att for i in range(layers)])
+
+
+def karopel(a, torch, Engine, SamplingParams) -> int:
+    """Prefill and decode throughput of Karopel layers of a real model's sizes beside Qwen3 layers of the same width."""
+    from dinfer_amd.config.karopel import KaropelConfig
+    shape = KAROPEL_SHAPES[a.karopel_shape]
+    layers = a.layers or 4
+    return beside_qwen3(a, torch, Engine, SamplingParams, "karopel", "Karopel", a.karopel_shape, shape,
+                        KaropelConfig.from_dict(karopel_config(shape, layers, 32768)))
+
+
 def kudurax(a, torch, Engine, SamplingParams) -> int:
     """Prefill and decode throughput of Kudurax layers of a real model's sizes beside Qwen3 layers of the same width
     (random weights, the same engine, the same steps): one JSON line with both."""
     from dinfer_amd.config.kudurax import KuduraxConfig
-    from dinfer_amd.config.qwen3 import Qwen3Config
     shape = KUDURAX_SHAPES[a.kudurax_shape]
+    layers = a.layers or 4
+    return beside_qwen3(a, torch, Engine, SamplingParams, "kudurax", "Kudurax", a.kudurax_shape, shape,
+                        KuduraxConfig.from_dict(kudurax_config(shape, layers, 32768)))
+
+
+def beside_qwen3(a, torch, Engine, SamplingParams, key: str, label: str, shape_name: str, shape: dict, config) -> int:
+    from dinfer_amd.config.qwen3 import Qwen3Config
     layers, vocab, page = a.layers or 4, 32768, 16
     PROMPT, CONTEXT = a.prompt, a.context
     batches = [b for b in (1, 8, 64) if b * CONTEXT <= 64 * 4096]
     models = {
-        "kudurax": KuduraxConfig.from_dict(kudurax_config(shape, layers, vocab)),
+        key: config,
         "qwen3": Qwen3Config.from_dict({**SIZES, "vocab_size": vocab, "hidden_size": shape["width"],
                                         "num_hidden_layers": layers, **shape["qwen"]}),
     }
@@ -286,13 +331,13 @@ def kudurax(a, torch, Engine, SamplingParams) -> int:
         result[name] = out
         del eng
         torch.cuda.empty_cache()
-    first = result.get("kudurax") or next(iter(result.values()))
+    first = result.get(key) or next(iter(result.values()))
     print(json.dumps({
-        "metric": f"decode tok/s (Kudurax layers of width {shape['width']}, batch 8, {PROMPT}-token prompts)",
+        "metric": f"decode tok/s ({label} layers of width {shape['width']}, batch 8, {PROMPT}-token prompts)",
         "value": first.get("decode_b8_tok_s"), "unit": "tokens/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
         "ms_per_step": first.get("decode_b8_ms"), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16" if a.dtype == "bfloat16" else "fp32", "data": "synthetic",
-        "config": {"model": f"Kudurax layers ({a.kudurax_shape}), random weights, beside Qwen3 layers of the same width",
+        "config": {"model": f"{label} layers ({shape_name}), random weights, beside Qwen3 layers of the same width",
                    "global_batch": 8, "seq_len": CONTEXT, "prompt_len": PROMPT, "parallelism": "single GPU",
                    "layers": layers, "vocab": vocab, "page_size": page, "hip_graph": not a.no_hip_graph, **shape},
         "models": result}))
@@ -314,13 +359,16 @@ def main() -> int:
     ap.add_argument("--prompt", type=int, default=DEFAULT_PROMPT, help="prompt tokens per request (and of the timed prefill)")
     ap.add_argument("--context", type=int, default=DEFAULT_CONTEXT, help="max_model_len the engine is built for")
     ap.add_argument("--kudurax-shape", default="2k", choices=sorted(KUDURAX_SHAPES), help="kudurax: layer sizes")
-    ap.add_argument("--only", default="", choices=["", "kudurax", "qwen3"], help="kudurax: measure one of the two models")
-    ap.add_argument("--workload", default="decode", choices=["decode", "serving", "closed", "kudurax"],
+    ap.add_argument("--karopel-shape", default="2k", choices=sorted(KAROPEL_SHAPES), help="karopel: layer sizes")
+    ap.add_argument("--only", default="", choices=["", "kudurax", "karopel", "qwen3"],
+                    help="kudurax, karopel: measure one of the two models")
+    ap.add_argument("--workload", default="decode", choices=["decode", "serving", "closed", "kudurax", "karopel"],
                     help="serving: 32 requests with prompts of 512 to 3,072 tokens fed in portions of 512 beside the "
                          "requests that decode, 256 outputs each (meant for the 14B shape); closed: --concurrency "
                          "requests live at any time, --prompt tokens in and --max-tokens out each, the load of the "
                          "reference's own serving bench without the server; kudurax: prefill and decode of Kudurax "
-                         "layers of a real model's sizes beside Qwen3 layers of the same width; each its own JSON line")
+                         "layers of a real model's sizes beside Qwen3 layers of the same width, karopel: the same for Karopel "
+                         "layers; each its own JSON line")
     ap.add_argument("--concurrency", type=int, default=8, help="closed: live requests")
     ap.add_argument("--max-tokens", type=int, default=128, help="closed: outputs per request")
     ap.add_argument("--num-requests", type=int, default=0, help="closed: requests in all (0: four per live request, at least 16)")
@@ -338,6 +386,8 @@ def main() -> int:
     from dinfer_amd.config.qwen3 import Qwen3Config
     if a.workload == "kudurax":
         return kudurax(a, torch, Engine, SamplingParams)
+    if a.workload == "karopel":
+        return karopel(a, torch, Engine, SamplingParams)
     if a.workload == "serving":
         return serving(a, torch, Engine, SamplingParams, Qwen3Config)
     if a.workload == "closed":

@@ -28,6 +28,11 @@
 //           over workgroups, each writing (m, l, o) partials; a merge kernel
 //           combines them.
 //
+// Options of the flash kernel (EXT; dinfer_attn_flash_ext, which serves single rows as well): the first keep_first
+// keys stay visible behind the window (one more short run of key blocks, walked by wave 0); a sink a head joins the
+// softmax's denominator when the waves' parts are combined; 2^(-slope_exp (h + 1) / H) times the distance is taken off
+// the scores (in raw score units, before the maximum); the output is multiplied by out_scale.
+//
 // Sizes: head_dim a multiple of 16 from the instantiated list, page size a
 // multiple of 8, G <= 16 for decode. Anything else is refused (the caller then
 // uses the plain kernel).
@@ -114,9 +119,11 @@ struct Frags {
 //   k_lo, k_hi  the keys this wave may touch at all (held pages, written slots)
 // load() issues the loads of one block, compute() consumes them; walk() keeps the next block's
 // loads in flight while the current one is computed.
-template <int DT, int NT, bool P2>
+template <int DT, int NT, bool P2, bool EXT = false>
 struct Tile {
   static constexpr int KS = (DT + 1) / 2;  // 32-wide steps over the head dimension
+  int keep_first = 0;      // EXT: keys below this stay visible whatever col_lo says
+  float slope_raw = 0.f;   // EXT: taken off a raw score per key of distance (the slope divided by the scale)
   static constexpr float LAZY = 6.f;       // weights up to 2^6 before the reference follows the maximum
   f32x4 o[NT][DT];
   float m[NT], l[NT];
@@ -229,10 +236,22 @@ struct Tile {
         x[r] = s[t][0][r];
         x[4 + r] = s[t][1][r];
       }
+      if (EXT) {
+        const float far = (float)(col_hi[t] - 1 - kg);   // the distance of the lane's first key from the column's position
+#pragma unroll
+        for (int e = 0; e < 8; ++e) x[e] = fmaf(-slope_raw, far - (float)e, x[e]);
+      }
       if (MASK) {
 #pragma unroll
-        for (int e = 0; e < 8; ++e)
-          if (kg + e < col_lo[t] || kg + e >= col_hi[t]) x[e] = -INFINITY;
+        for (int e = 0; e < 8; ++e) {
+          const int key = kg + e;
+          if (EXT) {
+            // (a kept key below the window may lie in a block of this run outside [k_lo, k_hi): its run comes later)
+            if ((key < col_lo[t] && key >= keep_first) || key >= col_hi[t] || key < k_lo || key >= k_hi) x[e] = -INFINITY;
+          } else if (key < col_lo[t] || key >= col_hi[t]) {
+            x[e] = -INFINITY;
+          }
+        }
       }
       float mx = x[0];
 #pragma unroll
@@ -340,12 +359,20 @@ struct Tile {
 // thousand workgroups of unequal length issued longest first, the chip stays evenly busy.
 // Measured on MI355X at head size 128 (one 2,048-token prompt, 32 heads): 122 us for the former
 // one-wave-per-tile kernel, where the longest tile set the time.
-template <int DT, int QT, bool P2>
+struct FlashExt {
+  int keep_first;       // with a window: keys below this stay visible
+  const float* sinks;   // [H] float or null
+  float slope_exp;      // 0: no distance bias
+  float out_scale;
+  float scale;          // the score scale itself (scale_log2e / log2(e))
+};
+
+template <int DT, int QT, bool P2, bool EXT = false>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 8))) attn_flash_kernel(
     const bf16* __restrict__ q, int64_t ld_q, bf16* __restrict__ out, int64_t ld_out, const bf16* __restrict__ kc,
     const bf16* __restrict__ vc, const int32_t* __restrict__ block_table, int64_t max_blocks,
     const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ seq_lens, int tiles_x, float scale_log2e,
-    int window, int H, int Hkv, int ps, int skip_single) {
+    int window, int H, int Hkv, int ps, int skip_single, FlashExt ext = FlashExt{}) {
   constexpr int D = DT * 16;
   constexpr int KS = (DT + 1) / 2;
   constexpr int QW = 16 * QT;  // query rows per workgroup
@@ -403,11 +430,25 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 8))
   const int k_lo = blk0 * 32 > all_lo ? blk0 * 32 : all_lo;
   const int k_hi = blk1 * 32 < all_hi ? blk1 * 32 : all_hi;
 
-  Tile<DT, QT, P2> tl;
+  Tile<DT, QT, P2, EXT> tl;
   tl.init(kc, vc, bt, (int)max_blocks, hk, Hkv, ps, k_lo, k_hi, scale_log2e);
+  if constexpr (EXT) {
+    tl.keep_first = window > 0 ? ext.keep_first : 0;
+    tl.slope_raw = ext.slope_exp != 0.f ? exp2f(-ext.slope_exp * (float)(h + 1) / (float)H) / ext.scale : 0.f;
+  }
   tl.template walk<true>(qf, col_lo, col_hi, [&](int kb) {
-    return kb + 31 > p_first || kb < all_lo || (window > 0 && kb < p_last - window + 1);
+    return kb + 31 > p_first || kb < all_lo || (window > 0 && kb < p_last - window + 1) || (EXT && kb + 32 > k_hi);
   });
+  if constexpr (EXT) {
+    // the kept first keys that the window of the tile's first row has passed: one more run, every block masked
+    const int kept = tl.keep_first < all_lo ? tl.keep_first : all_lo;
+    if (wave == 0 && kept > 0) {
+      tl.k_lo = 0;
+      tl.k_hi = kept;
+      tl.pages.init(bt, (int)max_blocks, ps, 0);
+      tl.template walk<false>(qf, col_lo, col_hi, [](int) { return true; });
+    }
+  }
 
   if (wave > 0) {
 #pragma unroll
@@ -443,8 +484,24 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 8))
       for (int d = 0; d < DT; ++d) tl.o[t][d] += part_o(r, t, d) * ar;
     }
     tl.l[t] = lsum;
-    const float lt = tl.sum_l(t);
-    const float inv = lt > 0.f ? 1.f / lt : 0.f;
+    float lt = tl.sum_l(t);
+    float inv;
+    if constexpr (EXT) {
+      float shrink = ext.out_scale;
+      if (ext.sinks) {  // one more term of the denominator, 2^(sink log2(e) - mc) against the parts' reference
+        const float d = ext.sinks[h] * LOG2E - mc;
+        if (d > 30.f) {  // a sink far above every score: the sums shrink instead of the term growing
+          const float f = exp2_raw(-d);
+          lt = lt * f + 1.f;
+          shrink *= f;
+        } else {
+          lt += exp2_raw(d);
+        }
+      }
+      inv = lt > 0.f ? shrink / lt : 0.f;
+    } else {
+      inv = lt > 0.f ? 1.f / lt : 0.f;
+    }
     const int row = q0 + t * 16 + i16;
     if (row < q_len) {
       bf16* op = out + (int64_t)(q_begin + row) * ld_out + (int64_t)h * D + 4 * g4;
@@ -857,10 +914,11 @@ __global__ void __launch_bounds__(64) attn_decode_merge_kernel(const float* __re
 
 inline bool aligned16(const void* p) { return ((uintptr_t)p % 16) == 0; }
 
-template <int DT>
+template <int DT, bool EXT = false>
 int launch_flash(const bf16* q, int64_t ld_q, bf16* out, int64_t ld_out, const bf16* kc, const bf16* vc,
                  const int32_t* bt, int64_t max_blocks, const int32_t* cu, const int32_t* sl, int num_reqs,
-                 int max_q_len, float scale, int window, int H, int Hkv, int ps, int skip_single, hipStream_t stream) {
+                 int max_q_len, float scale, int window, int H, int Hkv, int ps, int skip_single, hipStream_t stream,
+                 FlashExt ext = FlashExt{}) {
   const float sl2 = scale * LOG2E;
   const bool p2 = (ps & (ps - 1)) == 0;
   // 32 rows per workgroup where the head size leaves room for two row tiles (registers, and the LDS the
@@ -877,27 +935,27 @@ int launch_flash(const bf16* q, int64_t ld_q, bf16* out, int64_t ld_out, const b
     constexpr int QT = WIDE_OK ? 3 : 1;
     const int tiles = (max_q_len + 16 * QT - 1) / (16 * QT);
     if (wide_blocks > 0x7fffffff) return ERR_UNSUPPORTED;
-    auto kernel = p2 ? attn_flash_kernel<DT, QT, true> : attn_flash_kernel<DT, QT, false>;
+    auto kernel = p2 ? attn_flash_kernel<DT, QT, true, EXT> : attn_flash_kernel<DT, QT, false, EXT>;
     // (more than the 64 KB of LDS a launch may ask for without saying so)
     if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_of(QT)) != hipSuccess)
       return ERR_LAUNCH;
     kernel<<<(unsigned)wide_blocks, 256, lds_of(QT), stream>>>(q, ld_q, out, ld_out, kc, vc, bt, max_blocks, cu, sl, tiles,
-                                                              sl2, window, H, Hkv, ps, skip_single);
+                                                              sl2, window, H, Hkv, ps, skip_single, ext);
   } else if (DT <= 8 && max_q_len > 16) {
     constexpr int QT = DT <= 8 ? 2 : 1;
     const int tiles = (max_q_len + 16 * QT - 1) / (16 * QT);
     const int64_t blocks = (int64_t)tiles * H * num_reqs;
     if (blocks > 0x7fffffff) return ERR_UNSUPPORTED;
-    auto kernel = p2 ? attn_flash_kernel<DT, QT, true> : attn_flash_kernel<DT, QT, false>;
+    auto kernel = p2 ? attn_flash_kernel<DT, QT, true, EXT> : attn_flash_kernel<DT, QT, false, EXT>;
     kernel<<<(unsigned)blocks, 256, lds_of(QT), stream>>>(q, ld_q, out, ld_out, kc, vc, bt, max_blocks, cu, sl, tiles, sl2,
-                                                         window, H, Hkv, ps, skip_single);
+                                                         window, H, Hkv, ps, skip_single, ext);
   } else {
     const int tiles = (max_q_len + 15) / 16;
     const int64_t blocks = (int64_t)tiles * H * num_reqs;
     if (blocks > 0x7fffffff) return ERR_UNSUPPORTED;
-    auto kernel = p2 ? attn_flash_kernel<DT, 1, true> : attn_flash_kernel<DT, 1, false>;
+    auto kernel = p2 ? attn_flash_kernel<DT, 1, true, EXT> : attn_flash_kernel<DT, 1, false, EXT>;
     kernel<<<(unsigned)blocks, 256, lds_of(1), stream>>>(q, ld_q, out, ld_out, kc, vc, bt, max_blocks, cu, sl, tiles, sl2,
-                                                        window, H, Hkv, ps, skip_single);
+                                                        window, H, Hkv, ps, skip_single, ext);
   }
   return launch_status();
 }
@@ -994,6 +1052,26 @@ extern "C" int dinfer_attn_flash(const void* q, int64_t ld_q, void* out, int64_t
   DINFER_DISPATCH_HEAD_DIM(head_dim, return launch_flash<DT>(
       (const bf16*)q, ld_q, (bf16*)out, ld_out, (const bf16*)k_cache, (const bf16*)v_cache, block_table, max_blocks,
       cu_seqlens, seq_lens, num_reqs, max_q_len, scale, window, heads, kv_heads, page_size, skip_single, stream));
+}
+
+// The flash kernel with options, for prompt portions and single rows alike: keys below keep_first stay visible
+// behind the window; sinks [heads] float (or null) join the denominator; slope_exp E takes 2^(-E (h + 1) / heads)
+// times the distance off the scores; the output is multiplied by out_scale.
+extern "C" int dinfer_attn_flash_ext(const void* q, int64_t ld_q, void* out, int64_t ld_out, const void* k_cache,
+                                     const void* v_cache, const int32_t* block_table, int64_t max_blocks,
+                                     const int32_t* cu_seqlens, const int32_t* seq_lens, int num_reqs, int max_q_len,
+                                     float scale, int window, int keep_first, const float* sinks, float slope_exp,
+                                     float out_scale, int heads, int kv_heads, int head_dim, int page_size,
+                                     hipStream_t stream) {
+  if (num_reqs <= 0 || max_q_len <= 0) return OK;
+  if (!dinfer_attn_mfma_supports(head_dim, page_size, heads, kv_heads)) return ERR_UNSUPPORTED;
+  if (window < 0 || keep_first < 0 || !(scale > 0.f) || max_blocks <= 0 || ld_q % 8 || ld_out % 4 || !aligned16(q) ||
+      !aligned16(k_cache) || !aligned16(v_cache) || ((uintptr_t)out % 8))
+    return ERR_BAD_SHAPE;
+  const FlashExt ext{keep_first, sinks, slope_exp, out_scale, scale};
+  DINFER_DISPATCH_HEAD_DIM(head_dim, return (launch_flash<DT, true>(
+      (const bf16*)q, ld_q, (bf16*)out, ld_out, (const bf16*)k_cache, (const bf16*)v_cache, block_table, max_blocks,
+      cu_seqlens, seq_lens, num_reqs, max_q_len, scale, window, heads, kv_heads, page_size, 0, stream, ext)));
 }
 
 // Single-row requests only. cu_seqlens null: every request brings exactly one row (row b belongs to

@@ -63,6 +63,10 @@ SIGNATURES = {
         "attention",
         [_P, _L, _P, _L, _P, _P, _P, _L, _P, _P, _I, _I, _F, _I, _I, _I, _I, _I, _I, _P],
     ),
+    "dinfer_attn_flash_ext": (
+        "attention",
+        [_P, _L, _P, _L, _P, _P, _P, _L, _P, _P, _I, _I, _F, _I, _I, _P, _F, _F, _I, _I, _I, _I, _P],
+    ),
     "dinfer_attn_decode": (
         "attention",
         [_P, _L, _P, _L, _P, _L, _P, _P, _P, _L, _P, _P, _I, _I, _F, _I, _I, _I, _I, _I, _P],

@@ -656,6 +656,23 @@ def attn_flash(q, out, k_cache, v_cache, block_table, cu_seqlens, seq_lens, num_
     return out
 
 
+def attn_flash_ext(q, out, k_cache, v_cache, block_table, cu_seqlens, seq_lens, num_reqs: int, max_q_len: int, *,
+                   scale: float, window: int, heads: int, kv_heads: int, head_dim: int, page_size: int,
+                   keep_first: int = 0, sinks: torch.Tensor | None = None, slope_exp: float = 0.0,
+                   out_scale: float = 1.0) -> torch.Tensor:
+    """The matrix-core flash kernel with the options of attn_paged_ext (bfloat16, values of the keys' size, in value
+    pages), for prompt portions and single rows alike."""
+    _need_gpu(q, out, k_cache, v_cache, block_table, cu_seqlens, seq_lens, sinks)
+    _check_paged(q, out, k_cache, v_cache, block_table, seq_lens, num_reqs, heads, kv_heads, head_dim, page_size)
+    if sinks is not None:
+        assert sinks.dtype == torch.float32 and sinks.numel() == heads and sinks.is_contiguous()
+    lib.call("dinfer_attn_flash_ext", q.data_ptr(), _rows(q), out.data_ptr(), _rows(out), k_cache.data_ptr(),
+             v_cache.data_ptr(), block_table.data_ptr(), block_table.shape[1], cu_seqlens.data_ptr(), seq_lens.data_ptr(),
+             num_reqs, max_q_len, float(scale), int(window), int(keep_first), _ptr(sinks), float(slope_exp),
+             float(out_scale), heads, kv_heads, head_dim, page_size, _stream())
+    return out
+
+
 def attn_decode(q, out, part, k_cache, v_cache, block_table, cu_seqlens, seq_lens, num_reqs: int, splits: int, *,
                 scale: float, window: int, heads: int, kv_heads: int, head_dim: int, page_size: int):
     """Split-K attention for requests that bring one row. cu_seqlens None: row b is request b;

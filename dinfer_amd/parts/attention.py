@@ -63,6 +63,10 @@ class Attention(Mixer):
         self.qkv = Linear(hidden, self.q_size + self.kv_size + self.v_size)
         self.o = Linear(heads * self.v_dim, hidden)
         self.sinks = None
+        # decided in bind: the matrix-core flash kernel with options serves bfloat16 layers whose values have the keys'
+        # size; it reads values from transposed pages, so a layer whose values are its keys keeps them there as well
+        self.mfma_ext = False
+        self.stores_values = not self.values_are_keys
         self.position = POSITION_ENCODINGS.get(position.kind)(head_dim=head_dim, **position.params)
         self.q_norm = self.k_norm = None
         if qk_norm is not None:
@@ -70,8 +74,9 @@ class Attention(Mixer):
             self.q_norm, self.k_norm = cls(head_dim, **qk_norm.params), cls(head_dim, **qk_norm.params)
 
     def cache_spec(self):
+        # (asked after bind, which settles whether values that are the keys are stored a second time)
         return KVSpec(self.kv_heads, self.head_dim, self.window, v_dim=self.v_dim, keep_first=self.keep_first,
-                      values=not self.values_are_keys)
+                      values=self.stores_values)
 
     def tensors(self):
         D, Hd, nm = self.head_dim, self.hidden, self.names
@@ -129,6 +134,9 @@ class Attention(Mixer):
     def bind_core(self, ctx):
         self.page_size = ctx.page_size
         self.position.bind(ctx)
+        self.mfma_ext = bool(ctx.dtype == torch.bfloat16 and self.v_dim == self.head_dim
+                             and ops.attn_mfma_supports(self.head_dim, ctx.page_size, self.heads, self.kv_heads))
+        self.stores_values = not self.values_are_keys or self.mfma_ext
 
     def bind(self, ctx):
         ws = ctx.workspace
@@ -151,7 +159,7 @@ class Attention(Mixer):
         T = batch.num_tokens
         g = cache.group
         if self.extended or col or out_col:
-            return self._core_plain(qkv_buf, col, attn_buf, out_col, batch, cache)
+            return self._core_ext(qkv_buf, col, attn_buf, out_col, batch, cache)
         qn, pos = self.q_norm, self.position
         geometry = dict(heads=self.heads, kv_heads=self.kv_heads, head_dim=self.head_dim, q_off=0, k_off=self.q_size,
                         v_off=self.q_size + self.kv_size, positions=batch.positions, page_size=self.page_size)
@@ -188,21 +196,30 @@ class Attention(Mixer):
             window=self.window or 0, heads=self.heads, kv_heads=self.kv_heads, head_dim=self.head_dim,
             page_size=self.page_size)
 
-    def _core_plain(self, qkv_buf, col, attn_buf, out_col, batch, cache: CacheView):
-        """Per-head norm, rotation and cache write, then the plain kernel with this layer's options."""
+    def _core_ext(self, qkv_buf, col, attn_buf, out_col, batch, cache: CacheView):
+        """Per-head norm, rotation and cache write, then the flash kernel with this layer's options on the matrix
+        cores, or the plain kernel with them (32-bit, sizes the matrix-core kernel does not take)."""
         T, g = batch.num_tokens, cache.group
         qn, pos = self.q_norm, self.position
         if not pos.fused:
             raise NotImplementedError("attention with options takes a rotation by a table, or none")
         vd = self.v_dim
         ops.qkv_post(qkv_buf, T, heads=self.heads, kv_heads=self.kv_heads, head_dim=self.head_dim, q_off=col,
-                     k_off=col + self.q_size, v_off=col + self.q_size + (0 if self.values_are_keys else self.kv_size),
+                     k_off=col + self.q_size,     # (values that are the keys: the key columns as the product left them)
+                     v_off=col + self.q_size + (0 if self.values_are_keys else self.kv_size),
                      positions=batch.positions, page_size=self.page_size,
                      q_gain=qn.weight if qn else None, k_gain=self.k_norm.weight if qn else None,
                      eps=qn.eps if qn else 0.0, gain_offset=qn.weight_offset if qn else 0.0,
                      cos_sin=pos.table(), rotary_dim=pos.rotary_dim, rope_style=pos.style,
                      k_cache=cache.k, v_cache=cache.v, slot_mapping=batch.slot_mapping[g] if cache.owner else None,
                      token_runs=False, v_dim=vd)
+        if self.mfma_ext:
+            ops.attn_flash_ext(qkv_buf[:, col:], attn_buf[:, out_col:], cache.k, cache.v, batch.block_table[g],
+                               batch.cu_seqlens, batch.seq_lens, batch.num_reqs, batch.max_q_len, scale=self.scale,
+                               window=self.window or 0, heads=self.heads, kv_heads=self.kv_heads, head_dim=self.head_dim,
+                               page_size=self.page_size, keep_first=self.keep_first, sinks=self.sinks,
+                               slope_exp=self.slope_exp, out_scale=self.out_scale)
+            return
         ops.attn_paged_ext(qkv_buf[:, col:], attn_buf[:, out_col:], cache.k, cache.v, batch.block_table[g],
                            batch.cu_seqlens, batch.seq_lens, batch.num_reqs, T, scale=self.scale,
                            window=self.window or 0, heads=self.heads, kv_heads=self.kv_heads, head_dim=self.head_dim,

@@ -43,6 +43,8 @@ A2 = attention(3, 3, 40, 40, size=33, keep_first=0, base=300.0)                 
 P2 = parallel(2, 2, 24, 40, 3, 3, 40, 48, 2, 1.0, 1.0)                               # scales of one, two taps
 A3 = attention(8, 1, 32, 16, size=5, keep_first=6, scaling=dict(factor=8.0, low=1.0, high=4.0, original=16))   # keeps more than it sees
 P3 = parallel(6, 3, 8, 3, 2, 1, 64, 32, 4, 0.25, 2.0)
+A4 = attention(4, 2, 32, 32, size=24, keep_first=5, dims=16, scaling=BANDS)          # sizes the matrix-core kernel takes
+P4 = parallel(2, 1, 64, 9, 2, 1, 32, 32, 4, 0.7, 0.4)
 
 CONFIGS = {
     # layers 1 and 2 run three times; a layer without feed-forward; pages of 4
@@ -52,6 +54,9 @@ CONFIGS = {
     "C2": (model(131, 72, [with_mlp(A2, 64), with_mlp(P2, 40), with_mlp(A2, 88)], mult=1.0, logit_scale=1.7, eps=1e-3), 8, 12),
     # the whole model is one pass run twice, starting with a parallel layer; one tap would be no convolution: four
     "C3": (model(80, 48, [with_mlp(P3, 32), with_mlp(A3, 64)], loop=dict(start=0, stop=2, times=2), mult=0.3, logit_scale=0.5), 16, 13),
+    # bfloat16: both attentions on the matrix cores (heads of 32 and 64, pages of 8), the parallel layer looped
+    "C4": (model(120, 64, [with_mlp(A4, 96), with_mlp(P4, 64), with_mlp(A4, None)], loop=dict(start=1, stop=2, times=2),
+                 mult=0.4, logit_scale=1.3), 8, 14),
 }
 # one mechanism a model
 ONE = {
@@ -166,6 +171,20 @@ def test_one_mechanism(models, name, dtype):
 
 
 # ---- whole models ---------------------------------------------------------------------------------------------
+def test_which_attention_kernel_serves_which_model(models):
+    """bfloat16 with heads and pages the matrix-core kernel takes: that kernel, and values that are the keys are kept
+    in value pages as well; everything else: the plain kernel, keys only."""
+    for name, dtype, mfma in (("C4", "bfloat16", True), ("C4", "float32", False), ("C1", "bfloat16", False)):
+        r = make_runner(models, name, dtype)
+        mixers = [b.mixer for b in r.model.blocks]
+        plain_ones = [m for m in mixers if hasattr(m, "mfma_ext")]
+        joined = [m for mx in mixers if hasattr(mx, "members") for _, m, _, _ in mx.members if hasattr(m, "mfma_ext")]
+        assert plain_ones and joined and all(m.mfma_ext == mfma for m in plain_ones + joined)
+        assert all(m.stores_values == mfma for m in joined)
+        views = [v for v, b in zip(r.cache_views, [r.model.blocks[e.layer] for e in r.model.run]) if hasattr(b.mixer, "members")]
+        assert views and all(("left.v" in v.tensors) == mfma for v in views)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("name", NAMES)
 def test_whole_prompts(models, name, dtype):
@@ -433,6 +452,81 @@ def test_attention_with_options_alone(case, dtype):
         tol = 2e-5 if dtype == "float32" else 2e-2
         err = (out.double().cpu().view(H, V) - want).abs().max().item()
         assert err < tol * max(1.0, want.abs().max().item()), f"{case} target {target}: off by {err:.2e}"
+
+
+FLASH_CASES = [
+    # (heads, kv heads, dim, page, window, keep_first, sink, slope_exp, [(keys, rows of this step)])
+    (4, 2, 32, 8, 20, 5, True, 0.0, [(150, 37), (90, 1), (3, 3)]),
+    (4, 2, 64, 16, 40, 0, False, 8.0, [(200, 64), (41, 1)]),
+    (8, 1, 128, 16, 70, 12, True, 8.0, [(300, 100), (300, 1), (75, 2), (12, 12)]),
+    (3, 3, 48, 8, 0, 0, True, 0.0, [(100, 17), (64, 1)]),
+    (16, 4, 128, 16, 33, 40, True, 0.0, [(520, 130), (71, 1)]),     # keeps more than it sees; rows of three tiles
+]
+
+
+@pytest.mark.parametrize("kernel", ["flash", "plain"])
+@pytest.mark.parametrize("case", FLASH_CASES)
+def test_attention_with_options_on_the_matrix_cores(case, kernel):
+    """A step of prompt portions and single rows of several requests, pages shuffled among them: the matrix-core flash
+    kernel with options, and the plain kernel on the same bfloat16 caches, against float64. A row in eight is made to
+    look hard at one key: the oldest its window holds, the one before it, the last kept first key or the one after."""
+    from dinfer_amd.kernels import ops
+    H, G, D, page, window, keep, sink, slope_exp, reqs = case
+    g = torch.Generator().manual_seed(D + page)
+    sinks = (torch.randn(H, generator=g) * 2).float() if sink else None
+    scale = 0.9 / D ** 0.5
+    nb = sum(-(-n // page) for n, _ in reqs)
+    ids = list(range(nb + 2))
+    random.Random(D).shuffle(ids)
+    kp = torch.full((nb + 2, G, page, D), 7.0, dtype=torch.bfloat16)
+    vp = torch.full((nb + 2, G, page, D), 7.0, dtype=torch.bfloat16)
+    table = torch.full((len(reqs), max(-(-n // page) for n, _ in reqs)), -1, dtype=torch.int32)
+    qs, want, at = [], [], 0
+    for b, (n, rows) in enumerate(reqs):
+        k = torch.randn(G, n, D, generator=g).to(torch.bfloat16)
+        v = torch.randn(G, n, D, generator=g).to(torch.bfloat16)
+        for i in range(-(-n // page)):
+            table[b, i] = ids[at]
+            kp[ids[at], :, :min(page, n - i * page)] = k[:, i * page:(i + 1) * page]
+            vp[ids[at], :, :min(page, n - i * page)] = v[:, i * page:(i + 1) * page]
+            at += 1
+        for r in range(rows):
+            p = n - rows + r
+            q = torch.randn(H, D, generator=g)
+            if r % 8 == 0:
+                wlo = max(0, p - window + 1) if window else 0
+                target = [wlo, max(wlo - 1, 0), max(keep - 1, 0), min(keep, p)][(r // 8) % 4]
+                for h in range(H):
+                    kk = k[h // (H // G), target].float()
+                    q[h] += 5.0 * kk / kk.norm() * D ** 0.25
+            q = q.to(torch.bfloat16)
+            qs.append(q.view(H * D))
+            j = torch.arange(n)
+            mask = ((j <= p) & ((p - j < window) | (j < keep))) if window else (j <= p)
+            o = torch.zeros(H, D, dtype=F)
+            for h in range(H):
+                sc = (k[h // (H // G)].double() @ q[h].double()) * scale
+                if slope_exp:
+                    sc = sc - 2.0 ** (-slope_exp * (h + 1) / H) * (p - j).double()
+                o[h] = 0.5 * plain.softmax_rows(sc[None], mask[None], sinks[h].item() if sink else None)[0] @ v[h // (H // G)].double()
+            want.append(o.view(H * D))
+    q = torch.stack(qs).cuda()
+    T = q.shape[0]
+    out = torch.zeros(T, H * D, dtype=torch.bfloat16, device="cuda")
+    cu = torch.tensor([0] + list(torch.tensor([r for _, r in reqs]).cumsum(0)), dtype=torch.int32, device="cuda")
+    sl = torch.tensor([n for n, _ in reqs], dtype=torch.int32, device="cuda")
+    k_cache, v_cache = ops.k_cache_pack(kp).cuda(), vp.permute(0, 1, 3, 2).contiguous().cuda()
+    opts = dict(scale=scale, window=window, heads=H, kv_heads=G, head_dim=D, page_size=page, keep_first=keep,
+                sinks=sinks.cuda() if sink else None, slope_exp=slope_exp, out_scale=0.5)
+    if kernel == "flash":
+        assert ops.attn_mfma_supports(D, page, H, G)
+        ops.attn_flash_ext(q, out, k_cache, v_cache, table.cuda(), cu, sl, len(reqs), max(r for _, r in reqs), **opts)
+    else:
+        ops.attn_paged_ext(q, out, k_cache, v_cache, table.cuda(), cu, sl, len(reqs), T, **opts)
+    want = torch.stack(want)
+    err = (out.double().cpu() - want).abs().max(dim=1).values
+    worst = int(err.argmax())
+    assert err.max().item() < 2e-2 * max(1.0, want.abs().max().item()), f"{case}: row {worst} off by {err.max().item():.2e}"
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
