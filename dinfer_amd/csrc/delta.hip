@@ -8,9 +8,9 @@
 //
 //   delta_prep         one wave a (token, head of q, k or v): convolution over the step's rows and the request's
 //                      stored inputs, silu, unit norm of q and k; one more wave a token makes beta and g. Float out.
-//   delta_recurrence   the recurrence, token by token, for one request, one head and 32 columns of S a workgroup.
-//                      A thread owns a strip of rows of one column: lanes 0..7 of a group of eight share a column
-//                      and meet by three shuffles for each of the two products with S. k, q, v, beta and g of 16
+//   delta_recurrence   the recurrence, token by token, for one request, one head and 16 columns of S a workgroup.
+//                      A thread owns a strip of rows of one column: the 16 lanes of a DPP row share a column and
+//                      meet once a token, by four DPP additions for each of three sums. k, q, v, beta and g of 16
 //                      tokens wait in LDS while the next 16 are on their way in registers.
 //   delta_conv_update  moves the step's last taps - 1 inputs into the request's stored inputs (after prep has read
 //                      the old ones).
@@ -30,7 +30,7 @@ constexpr int WAVES = 4;
 constexpr int MAX_HEAD = 512;   // the largest D or V of the prep and out kernels (8 values a lane)
 constexpr int MAX_TAPS = 16;
 constexpr int CH = 16;          // tokens of a chunk in the recurrence
-constexpr int COLS = 32;        // columns of S a workgroup
+constexpr int COLS = 16;        // columns of S a workgroup
 
 __device__ __forceinline__ int request_of(const int32_t* __restrict__ cu, int num_reqs, int t) {
   int lo = 0, hi = num_reqs - 1;
@@ -131,19 +131,37 @@ __global__ void __launch_bounds__(256) delta_conv_update_kernel(const S* __restr
   }
 }
 
+// A lane's value plus that of the lane a DPP pattern pairs it with (full-rate vector instructions, no LDS).
+template <int CTRL>
+__device__ __forceinline__ float dpp_add(float v) {
+  return v + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+// The sum over a row of 16 lanes, in every lane of it: neighbours, pairs of a quad, the quads of a half row
+// (mirrored: all lanes of a quad hold the same sum by then), the two half rows.
+__device__ __forceinline__ float row16_sum(float v) {
+  v = dpp_add<0xB1>(v);    // quad_perm [1, 0, 3, 2]
+  v = dpp_add<0x4E>(v);    // quad_perm [2, 3, 0, 1]
+  v = dpp_add<0x141>(v);   // row_half_mirror
+  return dpp_add<0x140>(v);  // row_mirror
+}
+
+// One request, one head and COLS columns of S a workgroup; the 16 lanes of a DPP row share a column and own RPT
+// consecutive rows each (D <= 16 RPT). With a = S^T k, b = S^T q and c = k . q taken from the state before the
+// token, all three at once,   u = beta (v - g a),   o = g b + c u   (= (g S + k u^T)^T q),   S <- g S + k u^T:
+// one round of row sums a token instead of two, and no product waits for the state's update.
 template <int RPT>
 __global__ void __launch_bounds__(256) delta_recurrence_kernel(
     const float* __restrict__ work, int64_t ldw, float* __restrict__ state, const int32_t* __restrict__ slots,
     const int32_t* __restrict__ cu, const int32_t* __restrict__ seq_lens, float* __restrict__ out, int64_t ld_out,
     int G, int H, int D, int V) {
-  constexpr int DP = 8 * RPT;
-  __shared__ float ks[CH][DP];
-  __shared__ float qs[CH][DP];
+  constexpr int DP = 16 * RPT;
+  __shared__ __attribute__((aligned(16))) float ks[CH][DP];
+  __shared__ __attribute__((aligned(16))) float qs[CH][DP];
   __shared__ float vs[CH][COLS];
   __shared__ float bs[CH], gs[CH];
   const int b = blockIdx.x, h = blockIdx.y;
   const int tid = threadIdx.x;
-  const int rg = tid & 7, cj = tid >> 3;
+  const int rg = tid & 15, cj = tid >> 4;
   const int j = blockIdx.z * COLS + cj;
   const int t0 = cu[b], n = cu[b + 1] - t0;
   const int start = seq_lens[b] - n;
@@ -155,9 +173,9 @@ __global__ void __launch_bounds__(256) delta_recurrence_kernel(
 #pragma unroll
   for (int i = 0; i < RPT; ++i) S[i] = (start > 0 && col_ok && rg * RPT + i < D) ? sp[i] : 0.f;
 
-  // what a thread carries of the next chunk: RPT / 2 entries of k and of q, two of v, one of beta or g
+  // what a thread carries of the next chunk: RPT entries of k and of q, one of v, one of beta or g
   constexpr int PK = (CH * DP) / 256;
-  float pk[PK], pq[PK], pv[2], pbg = 0.f;
+  float pk[PK], pq[PK], pv = 0.f, pbg = 0.f;
   const float* wk = work + (int64_t)t0 * ldw;
   auto fetch = [&](int ct) {
 #pragma unroll
@@ -169,12 +187,10 @@ __global__ void __launch_bounds__(256) delta_recurrence_kernel(
       pk[e] = ok ? r[G * D] : 0.f;
       pq[e] = ok ? r[0] : 0.f;
     }
-#pragma unroll
-    for (int e = 0; e < 2; ++e) {
-      const int idx = tid + e * 256;
-      const int tok = idx / COLS, c = idx % COLS;
+    {
+      const int tok = tid / COLS, c = tid % COLS;
       const int col = blockIdx.z * COLS + c;
-      pv[e] = (ct + tok < n && col < V) ? wk[(int64_t)(ct + tok) * ldw + gd + h * V + col] : 0.f;
+      pv = (ct + tok < n && col < V) ? wk[(int64_t)(ct + tok) * ldw + gd + h * V + col] : 0.f;
     }
     if (tid < 2 * CH) {
       const int tok = tid % CH;
@@ -190,37 +206,37 @@ __global__ void __launch_bounds__(256) delta_recurrence_kernel(
       ks[idx / DP][idx % DP] = pk[e];
       qs[idx / DP][idx % DP] = pq[e];
     }
-#pragma unroll
-    for (int e = 0; e < 2; ++e) {
-      const int idx = tid + e * 256;
-      vs[idx / COLS][idx % COLS] = pv[e];
-    }
+    vs[tid / COLS][tid % COLS] = pv;
     if (tid < CH) bs[tid] = pbg;
     else if (tid < 2 * CH) gs[tid - CH] = pbg;
     __syncthreads();
     if (ct + CH < n) fetch(ct + CH);  // in flight while this chunk is worked through
     const int m = n - ct < CH ? n - ct : CH;
     for (int tok = 0; tok < m; ++tok) {
-      const float* kr = &ks[tok][rg * RPT];
-      const float* qr = &qs[tok][rg * RPT];
-      float dot = 0.f;
-#pragma unroll
-      for (int i = 0; i < RPT; ++i) dot = __builtin_fmaf(S[i], kr[i], dot);
-      dot += __shfl_xor(dot, 1, WAVE);
-      dot += __shfl_xor(dot, 2, WAVE);
-      dot += __shfl_xor(dot, 4, WAVE);
-      const float dec = gs[tok];
-      const float u = bs[tok] * (vs[tok][cj] - dec * dot);    // (g S)^T k = g (S^T k)
-      float o = 0.f;
+      float kr[RPT], qr[RPT];
 #pragma unroll
       for (int i = 0; i < RPT; ++i) {
-        S[i] = __builtin_fmaf(kr[i], u, dec * S[i]);
-        o = __builtin_fmaf(S[i], qr[i], o);
+        kr[i] = ks[tok][rg * RPT + i];
+        qr[i] = qs[tok][rg * RPT + i];
       }
-      o += __shfl_xor(o, 1, WAVE);
-      o += __shfl_xor(o, 2, WAVE);
-      o += __shfl_xor(o, 4, WAVE);
-      if (rg == 0 && col_ok) out[(int64_t)(t0 + ct + tok) * ld_out + h * V + j] = o;
+      float a0 = 0.f, a1 = 0.f, b0 = 0.f, b1 = 0.f, c0 = 0.f, c1 = 0.f;   // two chains a sum: a fixed order all the same
+#pragma unroll
+      for (int i = 0; i < RPT; i += 2) {
+        a0 = __builtin_fmaf(S[i], kr[i], a0);
+        b0 = __builtin_fmaf(S[i], qr[i], b0);
+        c0 = __builtin_fmaf(kr[i], qr[i], c0);
+        if (i + 1 < RPT) {
+          a1 = __builtin_fmaf(S[i + 1], kr[i + 1], a1);
+          b1 = __builtin_fmaf(S[i + 1], qr[i + 1], b1);
+          c1 = __builtin_fmaf(kr[i + 1], qr[i + 1], c1);
+        }
+      }
+      const float a = row16_sum(a0 + a1), bq = row16_sum(b0 + b1), c = row16_sum(c0 + c1);
+      const float dec = gs[tok];
+      const float u = bs[tok] * (vs[tok][cj] - dec * a);    // (g S)^T k = g (S^T k)
+#pragma unroll
+      for (int i = 0; i < RPT; ++i) S[i] = __builtin_fmaf(kr[i], u, dec * S[i]);
+      if (rg == 0 && col_ok) out[(int64_t)(t0 + ct + tok) * ld_out + h * V + j] = __builtin_fmaf(c, u, dec * bq);
     }
   }
   if (col_ok) {
@@ -309,10 +325,10 @@ extern "C" int dinfer_delta_recurrence(const float* work, int64_t ldw, float* st
 #define DELTA_REC(R_)                                                                                               \
   delta_recurrence_kernel<R_><<<grid, 256, 0, stream>>>(work, ldw, state, state_slots, cu_seqlens, seq_lens, out, \
                                                         ld_out, G, H, D, V)
-  if (D <= 32) DELTA_REC(4);
-  else if (D <= 64) DELTA_REC(8);
-  else if (D <= 128) DELTA_REC(16);
-  else DELTA_REC(32);
+  if (D <= 32) DELTA_REC(2);
+  else if (D <= 64) DELTA_REC(4);
+  else if (D <= 128) DELTA_REC(8);
+  else DELTA_REC(16);
 #undef DELTA_REC
   return launch_status();
 }
