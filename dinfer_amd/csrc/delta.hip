@@ -8,9 +8,9 @@
 //
 //   delta_prep         one wave a (token, head of q, k or v): convolution over the step's rows and the request's
 //                      stored inputs, silu, unit norm of q and k; one more wave a token makes beta and g. Float out.
-//   delta_recurrence   the recurrence, token by token, for one request, one head and 16 columns of S a workgroup.
-//                      A thread owns a strip of rows of one column: the 16 lanes of a DPP row share a column and
-//                      meet once a token, by four DPP additions for each of three sums. k, q, v, beta and g of 16
+//   delta_recurrence   the recurrence, token by token, for one request, one head and 8 columns of S a workgroup.
+//                      A thread owns a strip of rows of one column: the 32 lanes of half a wave share a column and
+//                      meet once a token, by four DPP additions and one exchange for each of three sums. k, q, v, beta and g of 16
 //                      tokens wait in LDS while the next 16 are on their way in registers.
 //   delta_conv_update  moves the step's last taps - 1 inputs into the request's stored inputs (after prep has read
 //                      the old ones).
@@ -30,7 +30,7 @@ constexpr int WAVES = 4;
 constexpr int MAX_HEAD = 512;   // the largest D or V of the prep and out kernels (8 values a lane)
 constexpr int MAX_TAPS = 16;
 constexpr int CH = 16;          // tokens of a chunk in the recurrence
-constexpr int COLS = 16;        // columns of S a workgroup
+constexpr int COLS = 8;         // columns of S a workgroup
 
 __device__ __forceinline__ int request_of(const int32_t* __restrict__ cu, int num_reqs, int t) {
   int lo = 0, hi = num_reqs - 1;
@@ -144,9 +144,16 @@ __device__ __forceinline__ float row16_sum(float v) {
   v = dpp_add<0x141>(v);   // row_half_mirror
   return dpp_add<0x140>(v);  // row_mirror
 }
+// The sum over 32 lanes (two DPP rows), in every lane of them.
+__device__ __forceinline__ float half_wave_sum(float v) {
+  v = row16_sum(v);
+  return v + __shfl_xor(v, 16, WAVE);
+}
 
-// One request, one head and COLS columns of S a workgroup; the 16 lanes of a DPP row share a column and own RPT
-// consecutive rows each (D <= 16 RPT). With a = S^T k, b = S^T q and c = k . q taken from the state before the
+// One request, one head and COLS columns of S a workgroup; the 32 lanes of half a wave share a column and own RPT
+// consecutive rows each (D <= 32 RPT): a wave's work a token is what bounds a prompt of one request, so a column is
+// spread over as many lanes as the sums' cost allows (16 lanes a column: 2,048 tokens of 16 heads of 128 x 128 in
+// 550 us; 8 lanes and the sums taken one after the other: 1,066 us). With a = S^T k, b = S^T q and c = k . q taken from the state before the
 // token, all three at once,   u = beta (v - g a),   o = g b + c u   (= (g S + k u^T)^T q),   S <- g S + k u^T:
 // one round of row sums a token instead of two, and no product waits for the state's update.
 template <int RPT>
@@ -154,14 +161,14 @@ __global__ void __launch_bounds__(256) delta_recurrence_kernel(
     const float* __restrict__ work, int64_t ldw, float* __restrict__ state, const int32_t* __restrict__ slots,
     const int32_t* __restrict__ cu, const int32_t* __restrict__ seq_lens, float* __restrict__ out, int64_t ld_out,
     int G, int H, int D, int V) {
-  constexpr int DP = 16 * RPT;
+  constexpr int DP = 32 * RPT;
   __shared__ __attribute__((aligned(16))) float ks[CH][DP];
   __shared__ __attribute__((aligned(16))) float qs[CH][DP];
   __shared__ float vs[CH][COLS];
   __shared__ float bs[CH], gs[CH];
   const int b = blockIdx.x, h = blockIdx.y;
   const int tid = threadIdx.x;
-  const int rg = tid & 15, cj = tid >> 4;
+  const int rg = tid & 31, cj = tid >> 5;
   const int j = blockIdx.z * COLS + cj;
   const int t0 = cu[b], n = cu[b + 1] - t0;
   const int start = seq_lens[b] - n;
@@ -187,7 +194,7 @@ __global__ void __launch_bounds__(256) delta_recurrence_kernel(
       pk[e] = ok ? r[G * D] : 0.f;
       pq[e] = ok ? r[0] : 0.f;
     }
-    {
+    if (tid < CH * COLS) {
       const int tok = tid / COLS, c = tid % COLS;
       const int col = blockIdx.z * COLS + c;
       pv = (ct + tok < n && col < V) ? wk[(int64_t)(ct + tok) * ldw + gd + h * V + col] : 0.f;
@@ -206,19 +213,28 @@ __global__ void __launch_bounds__(256) delta_recurrence_kernel(
       ks[idx / DP][idx % DP] = pk[e];
       qs[idx / DP][idx % DP] = pq[e];
     }
-    vs[tid / COLS][tid % COLS] = pv;
+    if (tid < CH * COLS) vs[tid / COLS][tid % COLS] = pv;
     if (tid < CH) bs[tid] = pbg;
     else if (tid < 2 * CH) gs[tid - CH] = pbg;
     __syncthreads();
     if (ct + CH < n) fetch(ct + CH);  // in flight while this chunk is worked through
     const int m = n - ct < CH ? n - ct : CH;
-    for (int tok = 0; tok < m; ++tok) {
-      float kr[RPT], qr[RPT];
+    // a token's operands are read from LDS while the token before is worked through
+    float kr[RPT], qr[RPT], vt, bt_, gt;
+    auto read = [&](int tok, float (&k_)[RPT], float (&q_)[RPT], float& v_, float& b_, float& g_) {
 #pragma unroll
       for (int i = 0; i < RPT; ++i) {
-        kr[i] = ks[tok][rg * RPT + i];
-        qr[i] = qs[tok][rg * RPT + i];
+        k_[i] = ks[tok][rg * RPT + i];
+        q_[i] = qs[tok][rg * RPT + i];
       }
+      v_ = vs[tok][cj];
+      b_ = bs[tok];
+      g_ = gs[tok];
+    };
+    read(0, kr, qr, vt, bt_, gt);
+    for (int tok = 0; tok < m; ++tok) {
+      float kn[RPT], qn[RPT], vn, bn, gn;
+      read(tok + 1 < m ? tok + 1 : tok, kn, qn, vn, bn, gn);
       float a0 = 0.f, a1 = 0.f, b0 = 0.f, b1 = 0.f, c0 = 0.f, c1 = 0.f;   // two chains a sum: a fixed order all the same
 #pragma unroll
       for (int i = 0; i < RPT; i += 2) {
@@ -231,12 +247,19 @@ __global__ void __launch_bounds__(256) delta_recurrence_kernel(
           c1 = __builtin_fmaf(kr[i + 1], qr[i + 1], c1);
         }
       }
-      const float a = row16_sum(a0 + a1), bq = row16_sum(b0 + b1), c = row16_sum(c0 + c1);
-      const float dec = gs[tok];
-      const float u = bs[tok] * (vs[tok][cj] - dec * a);    // (g S)^T k = g (S^T k)
+      const float a = half_wave_sum(a0 + a1), bq = half_wave_sum(b0 + b1), c = half_wave_sum(c0 + c1);
+      const float u = bt_ * (vt - gt * a);    // (g S)^T k = g (S^T k)
 #pragma unroll
-      for (int i = 0; i < RPT; ++i) S[i] = __builtin_fmaf(kr[i], u, dec * S[i]);
-      if (rg == 0 && col_ok) out[(int64_t)(t0 + ct + tok) * ld_out + h * V + j] = __builtin_fmaf(c, u, dec * bq);
+      for (int i = 0; i < RPT; ++i) S[i] = __builtin_fmaf(kr[i], u, gt * S[i]);
+      if (rg == 0 && col_ok) out[(int64_t)(t0 + ct + tok) * ld_out + h * V + j] = __builtin_fmaf(c, u, gt * bq);
+#pragma unroll
+      for (int i = 0; i < RPT; ++i) {
+        kr[i] = kn[i];
+        qr[i] = qn[i];
+      }
+      vt = vn;
+      bt_ = bn;
+      gt = gn;
     }
   }
   if (col_ok) {
@@ -325,10 +348,10 @@ extern "C" int dinfer_delta_recurrence(const float* work, int64_t ldw, float* st
 #define DELTA_REC(R_)                                                                                               \
   delta_recurrence_kernel<R_><<<grid, 256, 0, stream>>>(work, ldw, state, state_slots, cu_seqlens, seq_lens, out, \
                                                         ld_out, G, H, D, V)
-  if (D <= 32) DELTA_REC(2);
-  else if (D <= 64) DELTA_REC(4);
-  else if (D <= 128) DELTA_REC(8);
-  else DELTA_REC(16);
+  if (D <= 32) DELTA_REC(1);
+  else if (D <= 64) DELTA_REC(2);
+  else if (D <= 128) DELTA_REC(4);
+  else DELTA_REC(8);
 #undef DELTA_REC
   return launch_status();
 }
