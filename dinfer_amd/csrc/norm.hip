@@ -344,6 +344,122 @@ __global__ void __launch_bounds__(256) rmsnorm_stream_kernel(const void* __restr
     st_any(out, r * width + i, o_dt, row[i] * inv * (ld_any(w, i, p_dt) + off));
 }
 
+// The same for the combination the engine meets (float stream, float gains, branch and out of one type), widths that
+// are multiples of 8 up to 256 * 8 * ITERS: a thread keeps its 8-entry pieces in registers from the first read to the
+// last store and moves them 16 or 32 bytes at a time; the gains are asked for with the row, not after the sums.
+template <class SB, int ITERS>
+__global__ void __launch_bounds__(256) rmsnorm_stream_regs_kernel(const SB* __restrict__ branch, int64_t ld_b,
+                                                                  const float* __restrict__ wb, float eps_b, float off_b,
+                                                                  float mult, float* __restrict__ stream, int64_t ld_s,
+                                                                  const int32_t* __restrict__ rows,
+                                                                  const float* __restrict__ w, SB* __restrict__ out,
+                                                                  float eps, float off, int64_t width) {
+  __shared__ float red[16];
+  const int64_t r = blockIdx.x;
+  const int64_t s = rows ? (int64_t)rows[r] : r;
+  const int n8 = (int)(width / 8);
+  float x[ITERS][8], g[ITERS][8], y[ITERS][8];
+  float ss = 0.f;
+#pragma unroll
+  for (int it = 0; it < ITERS; ++it) {
+    const int i = it * 256 + threadIdx.x;
+    if (i < n8) {
+      const int64_t c = (int64_t)i * 8;
+      const f32x4 s0 = *(const f32x4*)(stream + s * ld_s + c), s1 = *(const f32x4*)(stream + s * ld_s + c + 4);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        x[it][j] = s0[j];
+        x[it][4 + j] = s1[j];
+      }
+      if (out) {
+        const f32x4 g0 = *(const f32x4*)(w + c), g1 = *(const f32x4*)(w + c + 4);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          g[it][j] = g0[j] + off;
+          g[it][4 + j] = g1[j] + off;
+        }
+      }
+      if (branch) {
+        const f32x4 b0 = *(const f32x4*)(wb + c), b1 = *(const f32x4*)(wb + c + 4);
+        float bv[8];
+        if constexpr (sizeof(SB) == 2) {
+          const bf16x8 p = *(const bf16x8*)(branch + s * ld_b + c);
+#pragma unroll
+          for (int j = 0; j < 8; ++j) bv[j] = (float)p[j];
+        } else {
+#pragma unroll
+          for (int j = 0; j < 8; ++j) bv[j] = to_f32(branch[s * ld_b + c + j]);
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const float v = bv[j];
+          y[it][j] = v * ((j < 4 ? b0[j] : b1[j - 4]) + off_b);
+          ss = add_square(ss, v);
+        }
+      }
+    }
+  }
+  if (branch) {
+    const float inv_b = 1.f / sqrtf(block_sum(ss, red) / (float)width + eps_b);
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+      const int i = it * 256 + threadIdx.x;
+      if (i < n8) {
+        const int64_t c = (int64_t)i * 8;
+        f32x4 s0, s1;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          x[it][j] = __builtin_fmaf(mult, y[it][j] * inv_b, x[it][j]);
+          if (j < 4) s0[j] = x[it][j]; else s1[j - 4] = x[it][j];
+        }
+        *(f32x4*)(stream + s * ld_s + c) = s0;
+        *(f32x4*)(stream + s * ld_s + c + 4) = s1;
+      }
+    }
+  }
+  if (!out) return;
+  ss = 0.f;
+#pragma unroll
+  for (int it = 0; it < ITERS; ++it) {
+    const int i = it * 256 + threadIdx.x;
+    if (i < n8) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) ss = add_square(ss, x[it][j]);
+    }
+  }
+  const float inv = 1.f / sqrtf(block_sum(ss, red) / (float)width + eps);
+#pragma unroll
+  for (int it = 0; it < ITERS; ++it) {
+    const int i = it * 256 + threadIdx.x;
+    if (i < n8) {
+      SB* o = out + r * width + (int64_t)i * 8;
+      if constexpr (sizeof(SB) == 2) {
+        bf16x8 p;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) p[j] = (bf16)(x[it][j] * inv * g[it][j]);
+        *(bf16x8*)o = p;
+      } else {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) o[j] = from_f32<SB>(x[it][j] * inv * g[it][j]);
+      }
+    }
+  }
+}
+
+template <class SB>
+void launch_stream_regs(const void* branch, int64_t ld_b, const void* wb, float eps_b, float off_b, float mult, void* stream_,
+                        int64_t ld_s, const int32_t* rows, const void* w, void* out, float eps, float off, int64_t n_rows,
+                        int64_t width, hipStream_t stream) {
+#define SN(IT)                                                                                                       \
+  rmsnorm_stream_regs_kernel<SB, IT><<<(unsigned)n_rows, 256, 0, stream>>>(                                          \
+      (const SB*)branch, ld_b, (const float*)wb, eps_b, off_b, mult, (float*)stream_, ld_s, rows, (const float*)w, \
+      (SB*)out, eps, off, width)
+  if (width <= 256 * 8) SN(1);
+  else if (width <= 256 * 8 * 2) SN(2);
+  else SN(4);
+#undef SN
+}
+
 }  // namespace
 
 // branch (may be null) [*, ld_b]; stream [*, ld_s], updated in place where a branch is given; out (may be null) dense
@@ -358,6 +474,17 @@ extern "C" int dinfer_rmsnorm_stream(const void* branch, int branch_dtype, int64
     return ERR_BAD_SHAPE;
   for (int dt : {branch_dtype, stream_dtype, param_dtype, out_dtype})
     if (dt != DT_F32 && dt != DT_BF16) return ERR_BAD_DTYPE;
+  // a float stream with float gains, branch and out of one type, rows of whole 16-byte pieces: rows in registers
+  const int io_dtype = branch ? branch_dtype : out_dtype;
+  if (stream_dtype == DT_F32 && param_dtype == DT_F32 && (!branch || !out || branch_dtype == out_dtype) &&
+      width % 8 == 0 && width <= 256 * 8 * 4 && ld_s % 4 == 0 && (!branch || ld_b % 8 == 0) && aligned16(stream_) &&
+      (!branch || (aligned16(branch) && aligned16(wb))) && (!out || (aligned16(out) && aligned16(w)))) {
+    if (io_dtype == DT_BF16)
+      launch_stream_regs<bf16>(branch, ld_b, wb, eps_b, off_b, mult, stream_, ld_s, rows, w, out, eps, off, n_rows, width, stream);
+    else
+      launch_stream_regs<float>(branch, ld_b, wb, eps_b, off_b, mult, stream_, ld_s, rows, w, out, eps, off, n_rows, width, stream);
+    return launch_status();
+  }
   if (width > 16384) return ERR_UNSUPPORTED;
   rmsnorm_stream_kernel<<<(unsigned)n_rows, 256, (size_t)width * sizeof(float), stream>>>(
       branch, branch_dtype, ld_b, wb, eps_b, off_b, mult, stream_, stream_dtype, ld_s, rows, w, param_dtype, out,

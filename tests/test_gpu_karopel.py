@@ -597,7 +597,7 @@ def test_delta_rule_kernels_alone(sizes, dtype):
         assert err < (1e-4 if dtype == "float32" else 3e-2) * max(1.0, want.abs().max().item()), f"request {r}: off by {err:.2e}"
 
 
-@pytest.mark.parametrize("width", [8, 72, 320, 4096, 5000])
+@pytest.mark.parametrize("width", [8, 10, 72, 320, 4096, 5000, 9000])
 @pytest.mark.parametrize("types", [("float32", "float32", "float32"), ("bfloat16", "float32", "bfloat16")])
 def test_stream_norm_kernel(width, types):
     """stream += mult * norm(branch) * (1 + wb); out = norm(stream) * (1 + w), with and without each half, on listed rows."""
