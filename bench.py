@@ -246,7 +246,7 @@ def karopel_config(shape: dict, layers: int, vocab: int) -> dict:
     att = dict(type="attention", mlp=dict(kind="dense", ff=shape["ff"]), mixer=dict(
         heads=shape["heads"], kv_heads=shape["kv_heads"], dim=d, vdim=d, scale=d ** -0.5,
         mask=dict(size=shape["window"], keep_first=shape["keep_first"]),
-        rot=dict(base=500000.0, dims=d, scaling=dict(factor=8.0, low=1.0, high=4.0, original=8192))))
+        rot=dict(base=1000000.0, dims=d, scaling=dict(factor=4.0, low=1.0, high=8.0, original=4096))))
     par = dict(type="parallel", mlp=dict(kind="dense", ff=shape["ff"]), mixer=dict(
         left=dict(heads=shape["left_heads"], kv_heads=shape["left_kv_heads"], dim=d, vdim=d, scale=d ** -0.5,
                   mask=dict(size=shape["left_window"])),

@@ -155,7 +155,7 @@ __device__ __forceinline__ float half_wave_sum(float v) {
 // spread over as many lanes as the sums' cost allows (16 lanes a column: 2,048 tokens of 16 heads of 128 x 128 in
 // 550 us; 8 lanes and the sums taken one after the other: 1,066 us). With a = S^T k, b = S^T q and c = k . q taken from the state before the
 // token, all three at once,   u = beta (v - g a),   o = g b + c u   (= (g S + k u^T)^T q),   S <- g S + k u^T:
-// one round of row sums a token instead of two, and no product waits for the state's update.
+// the rows are summed once a token instead of twice, and no product waits for the state's update.
 template <int RPT>
 __global__ void __launch_bounds__(256) delta_recurrence_kernel(
     const float* __restrict__ work, int64_t ldw, float* __restrict__ state, const int32_t* __restrict__ slots,

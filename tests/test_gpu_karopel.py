@@ -41,7 +41,7 @@ A1 = attention(4, 2, 16, 24, size=10, keep_first=3, dims=8, scaling=BANDS)      
 P1 = parallel(4, 1, 16, 7, 4, 2, 16, 8, 3, 0.6, 0.5)
 A2 = attention(3, 3, 40, 40, size=33, keep_first=0, base=300.0)                      # nothing kept, no scaling, odd head count
 P2 = parallel(2, 2, 24, 40, 3, 3, 40, 48, 2, 1.0, 1.0)                               # scales of one, two taps
-A3 = attention(8, 1, 32, 16, size=5, keep_first=6, scaling=dict(factor=8.0, low=1.0, high=4.0, original=16))   # keeps more than it sees
+A3 = attention(8, 1, 32, 16, size=5, keep_first=6, scaling=dict(factor=6.0, low=0.5, high=2.0, original=16))   # keeps more than it sees
 P3 = parallel(6, 3, 8, 3, 2, 1, 64, 32, 4, 0.25, 2.0)
 A4 = attention(4, 2, 32, 32, size=24, keep_first=5, dims=16, scaling=BANDS)          # sizes the matrix-core kernel takes
 P4 = parallel(2, 1, 64, 9, 2, 1, 32, 32, 4, 0.7, 0.4)
