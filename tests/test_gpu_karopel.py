@@ -648,3 +648,39 @@ def test_rotation_by_wavelength_bands(dims):
     want = plain.rotate_pairs(x[:, :32].double().view(5, 2, 16), pos, rot).view(5, 32)
     assert (buf[:, :32].double().cpu() - want).abs().max().item() < 1e-5
     assert torch.equal(buf[:, 32:].cpu(), x[:, 32:])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_trace_replay_program(models, tmp_path, dtype):
+    """bin/trace_run as a user runs it: a subprocess fed JSON lines; five requests through a pool made for three, so
+    pages and state slots are used again; logits read from the files it writes."""
+    import subprocess
+    import sys
+    from pathlib import Path
+    import numpy as np
+    d, cfg, w, page = models["C4"]
+    V = cfg["vocab"]
+    seqs = {k: tokens_for(cfg, n, sum(map(ord, k))) for k, n in (("a", 50), ("b", 90), ("c", 33), ("d", 64), ("e", 20))}
+    plan = [[("a", 30), ("b", 7)], [("a", 20), ("b", 2), ("c", 33)], [("b", 50)], [("b", 1), ("d", 40)],
+            [("b", 1), ("d", 2), ("e", 19)], [("b", 29), ("d", 22), ("e", 1)]]
+    steps, fed, expect = [], {k: 0 for k in seqs}, {}
+    for i, st in enumerate(plan):
+        entries, ends = [], []
+        for k, n in st:
+            wants = sorted({0, n - 1})
+            entries.append({"id": k, "tokens": seqs[k][fed[k]:fed[k] + n], "want": wants})
+            expect.setdefault(i, []).extend((k, fed[k] + j) for j in wants)
+            fed[k] += n
+            if fed[k] == len(seqs[k]):
+                ends.append(k)
+        steps.append({"step": i, "entries": entries, "end": ends})
+    root = Path(__file__).resolve().parent.parent
+    p = subprocess.run([sys.executable, str(root / "bin" / "trace_run"), "--model", str(d), "--dtype", dtype, "--out",
+                        str(tmp_path), "--max-tokens", "256", "--block-size", str(page)],
+                       input="".join(json.dumps(s) + "\n" for s in steps), capture_output=True, text=True, timeout=300)
+    assert p.returncode == 0, p.stderr[-2000:]
+    assert [l for l in p.stdout.splitlines() if l.startswith("done ")] == [f"done {i}" for i in range(len(plan))]
+    want = {k: plain.forward(v, w, cfg)[0] for k, v in seqs.items()}
+    for i, places in expect.items():
+        got = torch.from_numpy(np.fromfile(tmp_path / f"{i}.f32", dtype="<f4").reshape(len(places), V))
+        check_logits(got, torch.stack([want[k][pos] for k, pos in places]), dtype, f"replayed step {i}")
