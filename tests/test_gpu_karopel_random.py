@@ -1,0 +1,89 @@
+"""Karopel models drawn at random (sizes, head counts, layer order, windows, kept keys, taps, passes, pages), each
+replayed in mixed batches and in portions against the plain float64 model, in both dtypes: nothing in the engine may
+rest on the sizes of one model."""
+import json
+import random
+
+import pytest
+import torch
+
+import plain_karopel as plain
+from test_gpu_karopel import check_logits, compare_rows, cut, mixed_schedule, replay, tokens_for
+
+pytestmark = pytest.mark.gpu
+
+
+def draw_config(seed):
+    rng = random.Random(seed)
+    pick = rng.choice
+
+    def attention():
+        kv = pick([1, 2, 3])
+        dim = pick([8, 16, 24, 32, 40, 48, 64])
+        rot = None
+        if rng.random() < 0.9:
+            sc = None if rng.random() < 0.4 else dict(factor=pick([2.0, 8.0, 32.0]), low=pick([0.5, 1.0]), high=pick([2.0, 4.0]),
+                                                      original=pick([8, 32, 128]))
+            rot = dict(base=pick([100.0, 10000.0, 500000.0]), dims=pick([d for d in range(2, dim + 1, 2)]), scaling=sc)
+        return dict(heads=kv * pick([1, 2, 4]), kv_heads=kv, dim=dim, vdim=pick([dim, dim, 8, 16, 24, 32, 48]),
+                    scale=rng.uniform(0.5, 1.5) * dim ** -0.5,
+                    mask=dict(size=pick([1, 3, 8, 17, 40, 200]), keep_first=pick([0, 1, 4, 9, 50])), rot=rot)
+
+    def parallel():
+        kv, dim = pick([1, 2]), pick([8, 16, 32, 48, 64])
+        rkv = pick([1, 2])
+        return dict(left=dict(heads=kv * pick([1, 2, 4]), kv_heads=kv, dim=dim, vdim=dim, scale=rng.uniform(0.5, 1.5) * dim ** -0.5,
+                              mask=dict(size=pick([1, 2, 9, 30, 200]))),
+                    right=dict(heads=rkv * pick([1, 2, 3]), kv_heads=rkv, dim=pick([8, 16, 32, 48, 64, 96]),
+                               vdim=pick([8, 16, 24, 40, 64]), conv=pick([1, 2, 3, 4, 5])),
+                    left_scale=round(rng.uniform(0.2, 1.2), 3), right_scale=round(rng.uniform(0.2, 1.2), 3))
+
+    layers = []
+    for _ in range(rng.randint(2, 5)):
+        kind = pick(["attention", "parallel"])
+        layers.append(dict(type=kind, mixer=attention() if kind == "attention" else parallel(),
+                           mlp=None if rng.random() < 0.25 else dict(kind="dense", ff=pick([24, 40, 64]))))
+    loop = None
+    if rng.random() < 0.7:
+        start = rng.randrange(len(layers))
+        loop = dict(start=start, stop=rng.randint(start + 1, len(layers)), times=pick([1, 2, 3]))
+    cfg = dict(architecture="Karopel", vocab=rng.randint(50, 150), width=pick([32, 48, 64, 80]),
+               residual_mult=pick([0.3, 0.5, 1.0]), logit_scale=pick([0.5, 1.0, 2.0]), norm=dict(eps=pick([1e-6, 1e-5, 1e-3])),
+               loop=loop, layers=layers)
+    return cfg, pick([4, 8, 16])
+
+
+@pytest.fixture(scope="module")
+def drawn(tmp_path_factory):
+    from dinfer_amd.weights.safetensors_io import write_safetensors
+    out = {}
+    for seed in range(8):
+        cfg, page = draw_config(100 + seed)
+        d = tmp_path_factory.mktemp(f"karopel_r{seed}")
+        w = plain.random_weights(cfg, seed)
+        (d / "config.json").write_text(json.dumps(cfg))
+        write_safetensors(d / "model.safetensors", w, metadata={"format": "pt"})
+        out[seed] = (d, cfg, plain.as_float64(w), page)
+    return out
+
+
+def runner_for(drawn, seed, dtype, num_blocks, max_len=128):
+    from dinfer_amd.config import EngineOptions
+    from dinfer_amd.engine.runner import ModelRunner
+    d, _, _, page = drawn[seed]
+    opt = EngineOptions(dtype=dtype, max_model_len=max_len, max_num_seqs=4, max_num_batched_tokens=256, block_size=page,
+                        num_blocks=num_blocks, max_logits_rows=256, decode_exempt_from_budget=False, hip_graph=True)
+    return ModelRunner.from_dir(d, opt)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("seed", range(8))
+def test_drawn_model_in_mixed_batches_and_portions(drawn, seed, dtype):
+    _, cfg, w, page = drawn[seed]
+    toks, steps = mixed_schedule(cfg, seed)
+    r = runner_for(drawn, seed, dtype, num_blocks=4 * (96 // page) + 4, max_len=96)
+    compare_rows(replay(r, steps), cfg, w, toks, dtype, f"drawn model {seed}, mixed")
+    ids = tokens_for(cfg, 90, seed)
+    parts = cut(ids, [13, 2, 1, 1, 1, 30, 5])
+    rows = replay(r, [([("x", p, list(range(len(p))))], ["x"] if i == len(parts) - 1 else []) for i, p in enumerate(parts)])
+    compare_rows(rows, cfg, w, {"x": ids}, dtype, f"drawn model {seed}, portions")
