@@ -160,7 +160,11 @@ class DecoderModel:
         if self.embed_post is not None:
             self.embed_post[1].forward(self.hidden, T)
         if self.embedded is not None:
-            self.embedded[:T].copy_(self.hidden[:T])
+            if self.embed_post is None:     # gathered a second time: a kernel of the engine's own in a captured step
+                ops.embedding(batch.input_ids[:T], self.embed, self.embedded, getattr(batch, "feedback_src", None),
+                              getattr(batch, "last_tokens", None), scale=self.spec.embed_scale)
+            else:
+                self.embedded[:T].copy_(self.hidden[:T])
         pending = None
         for i, e in enumerate(self.run):
             block = self.blocks[e.layer]
