@@ -18,7 +18,7 @@
 //   out_scale      o is multiplied by it on store.
 //
 // K and V are read from the cache pages through the request's block table
-// (K page [Hkv][D / 8][page][8], V page [Hkv][D][page]); the step's own tokens were
+// (K page [Hkv][ceil(D / 8)][page][8], V page [Hkv][D][page]); the step's own tokens were
 // written there before this kernel runs.
 //
 // Reference behaviour: crates/kernels/cuda/gqa.cu:1037-1118 (plain paged
@@ -59,6 +59,7 @@ __global__ void __launch_bounds__(WAVES * 64) attn_paged_ref_kernel(
   const int first_key = window > 0 ? (p - window + 1 > 0 ? p - window + 1 : 0) : 0;
   const int32_t* bt = block_table + (int64_t)b * max_blocks;
   const int hk = live ? h / (H / Hkv) : 0;
+  const int Dp = (D + 7) & ~7;  // a head's keys fill whole 8-entry pieces of a page (the last one padded)
   const float slope = slope_exp != 0.f ? exp2f(-slope_exp * (float)(h + 1) / (float)H) : 0.f;
   // two runs of keys: the kept first ones that the window has passed, then the window itself
   const int kept = keep_first < first_key ? keep_first : first_key;
@@ -81,7 +82,7 @@ __global__ void __launch_bounds__(WAVES * 64) attn_paged_ref_kernel(
     float s = -INFINITY;
     if (live && j <= last) {
       const int blk = bt[j / page];
-      const S* kr = k_cache + ((int64_t)blk * Hkv + hk) * page * D;  // the head's page
+      const S* kr = k_cache + ((int64_t)blk * Hkv + hk) * page * Dp;  // the head's page
       const int off = j % page;
       float acc = 0.f;
       for (int d = 0; d < D; ++d) acc += qs[wave][d] * to_f32(kr[k_page_offset(off, d, page)]);
@@ -106,7 +107,7 @@ __global__ void __launch_bounds__(WAVES * 64) attn_paged_ref_kernel(
             const int key = j0 + jj;
             const int blk = bt[key / page];
             const S* vr = v_cache ? v_cache + (((int64_t)blk * Hkv + hk) * Dv + d) * page + (key % page)
-                                  : k_cache + ((int64_t)blk * Hkv + hk) * page * D + k_page_offset(key % page, d, page);
+                                  : k_cache + ((int64_t)blk * Hkv + hk) * page * Dp + k_page_offset(key % page, d, page);
             acc += ps[wave][jj] * to_f32(*vr);
           }
           o[c] = acc;

@@ -87,7 +87,8 @@ __global__ void __launch_bounds__(WAVES * 64) qkv_post_kernel(
   __syncthreads();  // the rotation reads partners that other lanes wrote
   if (!is_qk) return;
 
-  S* kd = (!is_q && slot >= 0) ? k_cache + (blk * Hkv + hk) * (int64_t)page * D : nullptr;  // the head's page
+  // (a head size that is no multiple of 8 fills its last 8-entry piece in part)
+  S* kd = (!is_q && slot >= 0) ? k_cache + (blk * Hkv + hk) * (int64_t)page * ((D + 7) & ~7) : nullptr;  // the head's page
   const float* cs = cos_sin ? cos_sin + (int64_t)pos[t] * rot : nullptr;
   const int half = rot / 2;
   for (int d = lane; d < D; d += 64) {
@@ -403,7 +404,7 @@ extern "C" int dinfer_qkv_post(int dtype, void* qkv, int64_t tokens, int64_t ld,
   if ((q_gain == nullptr) != (k_gain == nullptr)) return ERR_BAD_SHAPE;
   const int items = heads + 2 * kv_heads;
   const dim3 grid((unsigned)tokens, (unsigned)((items + WAVES - 1) / WAVES));
-  const bool whole_head_neox = style == 0 && head_dim % 2 == 0 && (!cos_sin || rotary_dim == head_dim) &&
+  const bool whole_head_neox = style == 0 && head_dim % 8 == 0 && (!cos_sin || rotary_dim == head_dim) &&
                                v_dim == head_dim && (v_cache || !slot_mapping);
   const bool vec_ok = dtype == DT_BF16 && (head_dim == 64 || head_dim == 128 || head_dim == 256) && ld % 8 == 0 &&
                       q_off % 8 == 0 && k_off % 8 == 0 && v_off % 8 == 0 && ((uintptr_t)qkv % 16) == 0 &&

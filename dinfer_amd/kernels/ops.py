@@ -518,9 +518,9 @@ def moe_combine(y: torch.Tensor, share: torch.Tensor, top: int, shared: torch.Te
 # so the rows of an MFMA operand (consecutive keys, one piece) are read as contiguous memory.
 # V pages [blocks, kv_heads, D, page]: transposed, a row holds one dimension of a page's keys.
 def k_cache_shape(blocks: int, kv_heads: int, page_size: int, head_dim: int) -> tuple:
-    if head_dim % 8 != 0:
-        raise ValueError(f"head_dim {head_dim}: the cache stores keys in pieces of 8 elements")
-    return (blocks, kv_heads, head_dim // 8, page_size, 8)
+    """A head size that is no multiple of 8 leaves its last piece filled in part (the plain kernels take that; the
+    matrix-core kernels take whole pieces only)."""
+    return (blocks, kv_heads, -(-head_dim // 8), page_size, 8)
 
 
 def v_cache_shape(blocks: int, kv_heads: int, page_size: int, head_dim: int) -> tuple:
@@ -530,7 +530,9 @@ def v_cache_shape(blocks: int, kv_heads: int, page_size: int, head_dim: int) -> 
 def k_cache_pack(rows: torch.Tensor) -> torch.Tensor:
     """[blocks, kv_heads, page, D] (one row per key) -> the layout of K pages."""
     nb, hkv, page, d = rows.shape
-    return rows.view(nb, hkv, page, d // 8, 8).permute(0, 1, 3, 2, 4).contiguous()
+    if d % 8:       # the last piece is filled in part
+        rows = torch.cat([rows, rows.new_zeros(nb, hkv, page, 8 - d % 8)], dim=-1)
+    return rows.view(nb, hkv, page, -1, 8).permute(0, 1, 3, 2, 4).contiguous()
 
 
 def k_cache_rows(pages: torch.Tensor) -> torch.Tensor:

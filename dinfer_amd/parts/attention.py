@@ -39,9 +39,8 @@ class Attention(Mixer):
                  values_are_keys: bool = False, out_scale: float = 1.0, names: dict | None = None):
         if heads % kv_heads:
             raise ValueError(f"heads {heads} not divisible by kv_heads {kv_heads}")
-        if head_dim <= 0 or head_dim % 8 or head_dim > ops.MAX_HEAD_DIM:   # said at build, not at the first step
-            raise ValueError(f"attention: head_dim {head_dim} has no kernel (multiples of 8 up to {ops.MAX_HEAD_DIM}; "
-                             "the cache stores keys in pieces of 8 elements)")
+        if head_dim <= 0 or head_dim > ops.MAX_HEAD_DIM:   # said at build, not at the first step
+            raise ValueError(f"attention: head_dim {head_dim} has no kernel (up to {ops.MAX_HEAD_DIM})")
         self.hidden, self.heads, self.kv_heads, self.head_dim = hidden, heads, kv_heads, head_dim
         self.window = window
         self.scale = float(scale) if scale is not None else head_dim ** -0.5

@@ -45,6 +45,8 @@ A3 = attention(8, 1, 32, 16, size=5, keep_first=6, scaling=dict(factor=6.0, low=
 P3 = parallel(6, 3, 8, 3, 2, 1, 64, 32, 4, 0.25, 2.0)
 A4 = attention(4, 2, 32, 32, size=24, keep_first=5, dims=16, scaling=BANDS)          # sizes the matrix-core kernel takes
 P4 = parallel(2, 1, 64, 9, 2, 1, 32, 32, 4, 0.7, 0.4)
+A5 = attention(2, 1, 20, 28, size=11, keep_first=2, dims=10)                         # head sizes that are no multiples of 8
+P5 = parallel(3, 3, 12, 6, 2, 2, 20, 10, 3, 0.8, 0.9)
 
 CONFIGS = {
     # layers 1 and 2 run three times; a layer without feed-forward; pages of 4
@@ -57,6 +59,7 @@ CONFIGS = {
     # bfloat16: both attentions on the matrix cores (heads of 32 and 64, pages of 8), the parallel layer looped
     "C4": (model(120, 64, [with_mlp(A4, 96), with_mlp(P4, 64), with_mlp(A4, None)], loop=dict(start=1, stop=2, times=2),
                  mult=0.4, logit_scale=1.3), 8, 14),
+    "C5": (model(77, 40, [with_mlp(A5, 56), with_mlp(P5, 24)], mult=0.6), 4, 15),
 }
 # one mechanism a model
 ONE = {
@@ -401,6 +404,8 @@ ATTN_CASES = [
     (4, 2, 16, 16, 8, 150, 20, 0, False, 8.0, True),
     (3, 3, 40, 8, 16, 200, 0, 0, True, 0.0, False),      # no window
     (8, 1, 32, 32, 4, 90, 7, 12, True, 8.0, False),       # keeps more than the window holds
+    (2, 1, 20, 12, 4, 70, 9, 2, True, 0.0, False),        # a head size that is no multiple of 8
+    (4, 2, 36, 36, 8, 70, 9, 0, False, 8.0, True),
 ]
 
 
