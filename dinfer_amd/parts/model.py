@@ -175,7 +175,10 @@ class DecoderModel:
                 elif pending is not None:
                     ops.add_rows(self.hidden, T, a=pending)
                     pending = None
-                self.before[i].forward(self.hidden, T, embedding=self.embedded)
+                if getattr(self.before[i], "needs_embedding", False):
+                    self.before[i].forward(self.hidden, T, embedding=self.embedded)
+                else:
+                    self.before[i].forward(self.hidden, T)
             # the input norm of the block that runs next, if that block lets the one before carry it (and nothing
             # touches the stream between the two)
             if block.carries_norms and i + 1 < len(self.run) and self.before[i + 1] is None:
