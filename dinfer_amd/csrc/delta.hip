@@ -108,6 +108,81 @@ __global__ void __launch_bounds__(WAVES * 64) delta_prep_kernel(
   }
 }
 
+// The same for head sizes that fill lanes evenly (D / 8 a power of two from 4 to 64 lanes, V a multiple of 8): a lane
+// takes 8 consecutive channels of a head (16-byte loads of the step's rows, the taps from a table transposed to
+// [K][channels]), the D / 8 lanes of a q or k head meet by shuffles for the unit norm, and a lane stores 32 bytes.
+// Lanes beyond the channels make beta and g. One workgroup covers 2,048 channels of a token.
+template <class S>
+__global__ void __launch_bounds__(256) delta_prep_vec_kernel(
+    const S* __restrict__ proj, int64_t ld, int64_t qkv_off, int64_t b_off, int64_t a_off,
+    const float* __restrict__ taps_t, const float* __restrict__ a_log, const float* __restrict__ dt_bias,
+    const S* __restrict__ conv_state, const int32_t* __restrict__ slots, const int32_t* __restrict__ cu,
+    const int32_t* __restrict__ seq_lens, float* __restrict__ work, int64_t ldw, int num_reqs, int G, int H, int D,
+    int V, int K, float eps, float q_scale) {
+  const int t = blockIdx.x;
+  const int gd = 2 * G * D, C = gd + H * V;
+  const int piece = blockIdx.y * 256 + threadIdx.x;   // which 8 channels
+  const int b = request_of(cu, num_reqs, t);
+  const int i = t - cu[b];
+  const int start = seq_lens[b] - (cu[b + 1] - cu[b]);
+  const S* row = proj + (int64_t)t * ld;
+  float* wr = work + (int64_t)t * ldw;
+  const int c = piece * 8;
+  if (c >= C) {   // the lanes behind the channels: step sizes and decays
+    const int h = c / 8 - C / 8;
+    if (h < H) {
+      wr[C + h] = sigmoid_f(to_f32(row[b_off + h]));
+      const float sp = softplus_f(to_f32(row[a_off + h]) + dt_bias[h]);
+      wr[C + H + h] = expf(-expf(a_log[h]) * sp);
+    }
+    return;
+  }
+  const S* old = (K > 1 && start > 0) ? conv_state + (int64_t)slots[b] * C * (K - 1) : nullptr;
+  float acc[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+  for (int j = K - 1; j >= 0; --j) {   // the oldest input first
+    float x[8];
+    if (i - j >= 0) {
+      const S* p = row + qkv_off + c - (int64_t)j * ld;
+      if constexpr (sizeof(S) == 2) {
+        const bf16x8 v = *(const bf16x8*)p;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) x[e] = (float)v[e];
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) x[e] = to_f32(p[e]);
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) x[e] = old ? to_f32(old[(int64_t)(c + e) * (K - 1) + (K - 1 + i - j)]) : 0.f;
+    }
+    const float* tp = taps_t + (int64_t)(K - 1 - j) * C + c;
+    const f32x4 w0 = *(const f32x4*)tp, w1 = *(const f32x4*)(tp + 4);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] = __builtin_fmaf(e < 4 ? w0[e] : w1[e - 4], x[e], acc[e]);
+  }
+  float ss = 0.f;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    acc[e] = silu_f(acc[e]);
+    ss = __builtin_fmaf(acc[e], acc[e], ss);
+  }
+  float mul = 1.f;
+  if (c < gd) {   // a q or k head: D / 8 neighbouring lanes, aligned to their count
+    for (int o = D / 16; o > 0; o >>= 1) ss += __shfl_xor(ss, o, WAVE);
+    mul = (c < G * D ? q_scale : 1.f) / sqrtf(ss + eps);
+  }
+  f32x4 o0, o1;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    o0[e] = acc[e] * mul;
+    o1[e] = acc[4 + e] * mul;
+  }
+  *(f32x4*)(wr + c) = o0;
+  *(f32x4*)(wr + c + 4) = o1;
+}
+
 template <class S>
 __global__ void __launch_bounds__(256) delta_conv_update_kernel(const S* __restrict__ proj, int64_t ld, int64_t qkv_off,
                                                                 S* __restrict__ conv_state,
@@ -306,15 +381,28 @@ __global__ void __launch_bounds__(WAVES * 64) delta_out_kernel(const float* __re
 // token's. a_log, dt_bias [H] float. conv_state [slots, 2 G D + H V, K - 1] in the step's dtype (unused with K = 1).
 // work [T, ldw] float, ldw >= 2 G D + H V + 2 H.
 extern "C" int dinfer_delta_prep(int dtype, const void* proj, int64_t ld, int64_t qkv_off, int64_t b_off, int64_t a_off,
-                                 const float* taps, const float* a_log, const float* dt_bias, const void* conv_state,
-                                 const int32_t* state_slots, const int32_t* cu_seqlens, const int32_t* seq_lens,
-                                 float* work, int64_t ldw, int num_reqs, int64_t tokens, int G, int H, int D, int V,
-                                 int K, float eps, float q_scale, hipStream_t stream) {
+                                 const float* taps, const float* taps_t, const float* a_log, const float* dt_bias,
+                                 const void* conv_state, const int32_t* state_slots, const int32_t* cu_seqlens,
+                                 const int32_t* seq_lens, float* work, int64_t ldw, int num_reqs, int64_t tokens, int G,
+                                 int H, int D, int V, int K, float eps, float q_scale, hipStream_t stream) {
+  // taps_t (may be null): the taps once more as [K, channels], for the kernel that takes 8 channels a lane
   if (tokens <= 0 || num_reqs <= 0) return OK;
   if (G <= 0 || H <= 0 || H % G || D <= 0 || V <= 0 || K <= 0 || tokens > 0x7fffffff ||
       ldw < 2 * (int64_t)G * D + (int64_t)H * V + 2 * H)
     return ERR_BAD_SHAPE;
   if (D > MAX_HEAD || V > MAX_HEAD || K > MAX_TAPS) return ERR_UNSUPPORTED;
+  const bool lanes_even = D >= 32 && D <= 512 && (D & (D - 1)) == 0 && V % 8 == 0;
+  if (taps_t && lanes_even && ld % 8 == 0 && qkv_off % 8 == 0 && ldw % 4 == 0 && ((uintptr_t)proj % 16) == 0 &&
+      ((uintptr_t)work % 16) == 0 && ((uintptr_t)taps_t % 16) == 0) {
+    const int pieces = (2 * G * D + H * V) / 8 + H;
+    const dim3 grid((unsigned)tokens, (unsigned)((pieces + 255) / 256));
+    DINFER_DISPATCH_DTYPE(dtype, {
+      delta_prep_vec_kernel<S><<<grid, 256, 0, stream>>>((const S*)proj, ld, qkv_off, b_off, a_off, taps_t, a_log, dt_bias,
+                                                         (const S*)conv_state, state_slots, cu_seqlens, seq_lens, work,
+                                                         ldw, num_reqs, G, H, D, V, K, eps, q_scale);
+    });
+    return launch_status();
+  }
   const dim3 grid((unsigned)tokens, (unsigned)((2 * G + H + 1 + WAVES - 1) / WAVES));
   DINFER_DISPATCH_DTYPE(dtype, {
     delta_prep_kernel<S><<<grid, WAVES * 64, 0, stream>>>((const S*)proj, ld, qkv_off, b_off, a_off, taps, a_log,

@@ -53,8 +53,8 @@ SIGNATURES = {
     "dinfer_rmsnorm_stream": ("norm", [_P, _I, _L, _P, _F, _F, _F, _P, _I, _L, _P, _P, _I, _P, _I, _F, _F, _L, _L, _P]),
     "dinfer_axpby": ("elementwise", [_I, _P, _L, _F, _P, _L, _F, _P, _L, _L, _L, _P]),
     "dinfer_add_rows": ("elementwise", [_P, _I, _L, _P, _I, _L, _P, _I, _L, _L, _P]),
-    "dinfer_delta_prep": ("delta", [_I, _P, _L, _L, _L, _L, _P, _P, _P, _P, _P, _P, _P, _P, _L, _I, _L, _I, _I, _I, _I,
-                                    _I, _F, _F, _P]),
+    "dinfer_delta_prep": ("delta", [_I, _P, _L, _L, _L, _L, _P, _P, _P, _P, _P, _P, _P, _P, _P, _L, _I, _L, _I, _I, _I,
+                                    _I, _I, _F, _F, _P]),
     "dinfer_delta_conv_update": ("delta", [_I, _P, _L, _L, _P, _P, _P, _P, _I, _I, _I, _P]),
     "dinfer_delta_recurrence": ("delta", [_P, _L, _P, _P, _P, _P, _P, _L, _I, _I, _I, _I, _I, _P]),
     "dinfer_delta_out": ("delta", [_I, _P, _L, _P, _L, _L, _P, _P, _L, _L, _L, _I, _I, _F, _F, _P]),

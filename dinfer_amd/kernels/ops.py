@@ -264,9 +264,10 @@ def delta_work_columns(qk_heads: int, heads: int, dim: int, vdim: int) -> int:
 def delta_prep(proj: torch.Tensor, tokens: int, *, qkv_off: int, b_off: int, a_off: int, taps: torch.Tensor,
                a_log: torch.Tensor, dt_bias: torch.Tensor, conv_state: torch.Tensor | None, state_slots: torch.Tensor,
                cu_seqlens: torch.Tensor, seq_lens: torch.Tensor, work: torch.Tensor, num_reqs: int, qk_heads: int,
-               heads: int, dim: int, vdim: int, eps: float, q_scale: float) -> None:
+               heads: int, dim: int, vdim: int, eps: float, q_scale: float, taps_t: torch.Tensor | None = None) -> None:
     """Short convolution (over the step's rows and the request's stored inputs), silu, unit q and k, step sizes and
-    decays: proj [T, *] -> work [T, delta_work_columns] float32."""
+    decays: proj [T, *] -> work [T, delta_work_columns] float32. taps_t: the taps transposed [K, channels]; with them
+    the kernel that takes 8 channels a lane serves the sizes it fits."""
     _need_gpu(proj, taps, a_log, dt_bias, conv_state, state_slots, cu_seqlens, seq_lens, work)
     C = 2 * qk_heads * dim + heads * vdim
     K = taps.shape[1]
@@ -277,8 +278,10 @@ def delta_prep(proj: torch.Tensor, tokens: int, *, qkv_off: int, b_off: int, a_o
     if K > 1:
         assert conv_state is not None and conv_state.dtype == proj.dtype and conv_state.is_contiguous()
         assert tuple(conv_state.shape[1:]) == (C, K - 1)
+    if taps_t is not None:
+        assert taps_t.dtype == torch.float32 and tuple(taps_t.shape) == (K, C) and taps_t.is_contiguous()
     lib.call("dinfer_delta_prep", dtype_code(proj.dtype), proj.data_ptr(), _rows(proj), qkv_off, b_off, a_off,
-             taps.data_ptr(), a_log.data_ptr(), dt_bias.data_ptr(), _ptr(conv_state) if K > 1 else None,
+             taps.data_ptr(), _ptr(taps_t), a_log.data_ptr(), dt_bias.data_ptr(), _ptr(conv_state) if K > 1 else None,
              state_slots.data_ptr(), cu_seqlens.data_ptr(), seq_lens.data_ptr(), work.data_ptr(), _rows(work), num_reqs,
              tokens, qk_heads, heads, dim, vdim, K, float(eps), float(q_scale), _stream())
 

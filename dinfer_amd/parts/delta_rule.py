@@ -90,6 +90,7 @@ class GatedDeltaRule(Mixer):
         n = self.names
         # small parameters in 32 bits (exact for a bfloat16 file): they enter the recurrence
         self.conv_taps = torch.cat([get(n[k]).float() for k in ("q_conv", "k_conv", "v_conv")], dim=0).contiguous()
+        self.conv_taps_t = self.conv_taps.t().contiguous()      # [taps, channels]: 8 channels' taps in one load
         self.a_log = get(n["A_log"]).float().contiguous()
         self.dt_bias = get(n["dt_bias"]).float().contiguous()
         self.norm_weight = get(n["norm"]).float().contiguous()
@@ -126,7 +127,7 @@ class GatedDeltaRule(Mixer):
         sizes = dict(qk_heads=self.qk_heads, heads=self.heads, dim=self.dim, vdim=self.vdim)
         ops.delta_prep(proj_buf, T, qkv_off=col, b_off=col + self.b_off, a_off=col + self.a_off, taps=self.conv_taps,
                        a_log=self.a_log, dt_bias=self.dt_bias, conv_state=cache.conv, work=self.work,
-                       eps=self.unit_eps, q_scale=self.dim ** -0.5, **common, **sizes)
+                       eps=self.unit_eps, q_scale=self.dim ** -0.5, taps_t=self.conv_taps_t, **common, **sizes)
         if cache.owner:
             ops.delta_conv_update(proj_buf, qkv_off=col, conv_state=cache.conv, **common)
         ops.delta_recurrence(self.work, cache.state, self.o_buf, **common, **sizes)

@@ -535,10 +535,13 @@ def test_attention_with_options_on_the_matrix_cores(case, kernel):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("sizes", [(2, 1, 8, 8, 2), (4, 2, 16, 24, 4), (3, 3, 40, 48, 3), (2, 1, 64, 32, 1), (2, 2, 128, 136, 4)])
-def test_delta_rule_kernels_alone(sizes, dtype):
+@pytest.mark.parametrize("wide_loads", [False, True])
+@pytest.mark.parametrize("sizes", [(2, 1, 8, 8, 2), (4, 2, 16, 24, 4), (3, 3, 40, 48, 3), (2, 1, 64, 32, 1), (2, 2, 128, 136, 4),
+                                   (6, 3, 32, 8, 5)])
+def test_delta_rule_kernels_alone(sizes, dtype, wide_loads):
     """Two requests of unequal length in one step, then each continued by portions and single rows, against the plain
-    recurrence over the whole sequences; slots are not the requests' order, and one starts in a slot that holds junk."""
+    recurrence over the whole sequences; slots are not the requests' order, and one starts in a slot that holds junk.
+    wide_loads: the transposed taps are given too, so sizes that fit it run the kernel that takes 8 channels a lane."""
     from dinfer_amd.kernels import ops
     H, G, D, V, K = sizes
     dt = getattr(torch, dtype)
@@ -568,7 +571,7 @@ def test_delta_rule_kernels_alone(sizes, dtype):
         common = dict(state_slots=ss, cu_seqlens=cu, seq_lens=sl, num_reqs=len(step))
         ops.delta_prep(rows, T, qkv_off=0, b_off=C + H * V, a_off=C + H * V + H, taps=taps.cuda(), a_log=a_log.cuda(),
                        dt_bias=dt_bias.cuda(), conv_state=conv, work=work, qk_heads=G, heads=H, dim=D, vdim=V, eps=1e-6,
-                       q_scale=D ** -0.5, **common)
+                       q_scale=D ** -0.5, taps_t=taps.t().contiguous().cuda() if wide_loads else None, **common)
         ops.delta_conv_update(rows, qkv_off=0, conv_state=conv, **common)
         ops.delta_recurrence(work, state, o, qk_heads=G, heads=H, dim=D, vdim=V, **common)
         out = torch.zeros(T, H * V, dtype=dt, device="cuda")
