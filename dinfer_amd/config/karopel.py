@@ -88,7 +88,9 @@ def _attention(m: dict, where: str, rotation: bool, keeps: bool) -> AttentionCon
         if not isinstance(rot, dict):
             raise ConfigError(f"config key {where}'rot' must be an object or null, got {rot!r}")
         kw["rot_base"] = _num(rot, "base", float, where + "rot.")
-        kw["rot_dims"] = _num(rot, "dims", int, where + "rot.")
+        kw["rot_dims"] = _num(rot, "dims", int, where + "rot.", positive=False)
+        if kw["rot_dims"] < 0:
+            raise ConfigError(f"config key {where}'rot.dims' must not be negative, got {kw['rot_dims']}")
         sc = rot.get("scaling")
         if sc is not None:
             if not isinstance(sc, dict):

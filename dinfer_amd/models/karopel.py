@@ -26,7 +26,7 @@ def _attention(cfg: KaropelConfig, a: AttentionConfig, plain_left: bool):
     if plain_left:
         return part("attention", heads=a.heads, kv_heads=a.kv_heads, head_dim=a.dim, position=part("none"), window=a.window,
                     scale=a.scale, slope_exp=SLOPE_EXP, values_are_keys=True, names=names)
-    if a.rot_base is None:
+    if a.rot_base is None or a.rot_dims == 0:      # no rotation, or one of no entries
         position = part("none")
     else:
         s = a.rot_scaling
