@@ -24,7 +24,7 @@ def draw_config(seed):
         if rng.random() < 0.9:
             sc = None if rng.random() < 0.4 else dict(factor=pick([2.0, 8.0, 32.0]), low=pick([0.5, 1.0]), high=pick([2.0, 4.0]),
                                                       original=pick([8, 32, 128]))
-            rot = dict(base=pick([100.0, 10000.0, 500000.0]), dims=pick([d for d in range(2, dim + 1, 2)]), scaling=sc)
+            rot = dict(base=pick([100.0, 10000.0, 250000.0]), dims=pick([d for d in range(2, dim + 1, 2)]), scaling=sc)
         return dict(heads=kv * pick([1, 2, 4]), kv_heads=kv, dim=dim, vdim=pick([dim, dim, 8, 16, 24, 32, 48]),
                     scale=rng.uniform(0.5, 1.5) * dim ** -0.5,
                     mask=dict(size=pick([1, 3, 8, 17, 40, 200]), keep_first=pick([0, 1, 4, 9, 50])), rot=rot)
@@ -48,7 +48,7 @@ def draw_config(seed):
         start = rng.randrange(len(layers))
         loop = dict(start=start, stop=rng.randint(start + 1, len(layers)), times=pick([1, 2, 3]))
     cfg = dict(architecture="Karopel", vocab=rng.randint(50, 150), width=pick([32, 48, 64, 80]),
-               residual_mult=pick([0.3, 0.5, 1.0]), logit_scale=pick([0.5, 1.0, 2.0]), norm=dict(eps=pick([1e-6, 1e-5, 1e-3])),
+               residual_mult=pick([0.25, 0.5, 1.0]), logit_scale=pick([0.5, 1.0, 1.5]), norm=dict(eps=pick([1e-6, 1e-5, 1e-3])),
                loop=loop, layers=layers)
     return cfg, pick([4, 8, 16])
 

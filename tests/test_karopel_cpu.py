@@ -20,11 +20,11 @@ def attention(size=10, keep=3, dims=8, scaling=None):
 def parallel(conv=3):
     return dict(type="parallel", mlp=None,
                 mixer=dict(left=dict(heads=4, kv_heads=1, dim=16, vdim=16, scale=0.25, mask=dict(size=7)),
-                           right=dict(heads=4, kv_heads=2, dim=16, vdim=8, conv=conv), left_scale=0.6, right_scale=0.5))
+                           right=dict(heads=4, kv_heads=2, dim=16, vdim=8, conv=conv), left_scale=0.7, right_scale=0.45))
 
 
 def config(**kw):
-    cfg = dict(architecture="Karopel", vocab=96, width=64, residual_mult=0.5, logit_scale=2.0, norm=dict(eps=1e-6),
+    cfg = dict(architecture="Karopel", vocab=96, width=64, residual_mult=0.5, logit_scale=1.5, norm=dict(eps=1e-5),
                loop=dict(start=1, stop=3, times=3), layers=[parallel(), attention(), attention(), parallel()])
     cfg.update(kw)
     return cfg
